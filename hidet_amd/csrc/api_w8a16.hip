@@ -1,0 +1,25 @@
+// Entry point of the W8A16 matmul: argument checks and the choice of kernel family.
+#include "common.h"
+
+namespace qmm {
+void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
+                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+}
+
+using namespace qmm;
+
+HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
+                                                   int64_t k, int64_t n, int64_t lda, int parallel_k_parts,
+                                                   void *workspace, int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
+    QMM_CHECK(lda >= k, "row stride of a (" << lda << ") is smaller than K (" << k << ")");
+    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    QMM_CHECK(parallel_k_parts >= 0, "parallel_k_parts must be >= 0");
+    if (m == 0 || n == 0) return;
+    QMM_CHECK(a && w && scale && c, "null tensor pointer");
+    QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);
+    QMM_ENTRY_END
+}

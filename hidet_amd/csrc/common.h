@@ -1,0 +1,132 @@
+// Shared host/device helpers for the quantized-matmul library (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <cstdint>
+#include <exception>
+#include <sstream>
+#include <string>
+
+#include "../../include/hidet_qmm.h"
+
+#define HIDET_API extern "C" __attribute__((visibility("default")))
+
+namespace qmm {
+
+// Thrown inside an entry point, turned into the thread-local last-error string at the boundary.
+struct Error : std::exception {
+    std::string msg;
+    explicit Error(std::string m) : msg(std::move(m)) {}
+    const char *what() const noexcept override { return msg.c_str(); }
+};
+
+struct Thrower {
+    std::ostringstream os;
+    Thrower(const char *file, int line) { os << file << ":" << line << ": "; }
+    [[noreturn]] void raise() { throw Error(os.str()); }
+};
+
+#define QMM_FAIL(...)                         \
+    do {                                      \
+        ::qmm::Thrower _t(__FILE__, __LINE__); \
+        _t.os << __VA_ARGS__;                 \
+        _t.raise();                           \
+    } while (0)
+
+#define QMM_CHECK(cond, ...)                  \
+    do {                                      \
+        if (!(cond)) QMM_FAIL(__VA_ARGS__);   \
+    } while (0)
+
+#define QMM_HIP(call)                                                                   \
+    do {                                                                                \
+        hipError_t _e = (call);                                                         \
+        if (_e != hipSuccess) QMM_FAIL(#call << " failed: " << hipGetErrorString(_e));  \
+    } while (0)
+
+// Body of every extern "C" entry point: nothing may propagate across the C boundary.
+#define QMM_ENTRY_BEGIN try {
+#define QMM_ENTRY_END                            \
+    }                                            \
+    catch (const std::exception &e) {            \
+        hidet_set_last_error(e.what());          \
+        return;                                  \
+    }                                            \
+    catch (...) {                                \
+        hidet_set_last_error("unknown error");   \
+        return;                                  \
+    }
+
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline size_t dtype_bytes(int dt) {
+    switch (dt) {
+        case HIDET_QMM_F32: return 4;
+        case HIDET_QMM_F16:
+        case HIDET_QMM_BF16:
+        case HIDET_QMM_I16: return 2;
+        case HIDET_QMM_I8:
+        case HIDET_QMM_E4M3: return 1;
+        default: QMM_FAIL("unknown dtype code " << dt);
+    }
+}
+
+// One-shot timing hook: when a (start, stop) event pair is armed on this thread, the next main
+// kernel launch records its own begin/end timestamps into them (hipExtLaunchKernelGGL).
+struct TimingSlot {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+TimingSlot &timing_slot();
+
+template <typename... KArgs, typename... Args>
+inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args) {
+    TimingSlot &ts = timing_slot();
+    if (ts.start != nullptr) {
+        hipEvent_t s = ts.start, e = ts.stop;
+        ts.start = ts.stop = nullptr;
+        hipExtLaunchKernelGGL(kernel, grid, block, shmem, stream, s, e, 0, static_cast<KArgs>(args)...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, shmem, stream, static_cast<KArgs>(args)...);
+    }
+    QMM_HIP(hipGetLastError());
+}
+
+// Helper kernels (fills, conversions) never consume the timing slot.
+template <typename... KArgs, typename... Args>
+inline void launch_aux(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args) {
+    hipLaunchKernelGGL(kernel, grid, block, shmem, stream, static_cast<KArgs>(args)...);
+    QMM_HIP(hipGetLastError());
+}
+
+// ---- device-side numeric helpers ---------------------------------------------------------------
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef int int8v_t __attribute__((ext_vector_type(8)));
+typedef int int4v_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
+
+// float32 -> bfloat16 bits, round to nearest even (NaN kept quiet)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    _Float16 h = static_cast<_Float16>(f);  // v_cvt_f16_f32: round to nearest even
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) { return static_cast<float>(__builtin_bit_cast(_Float16, b)); }
+
+}  // namespace qmm

@@ -1,0 +1,297 @@
+// Quantization kernels: symmetric int8/int16 quantize + dequantize over a [outer, reduce, inner]
+// view, group-wise signed int4 with nibble packing, and per-tensor float8 e4m3.
+//
+// Every division and rounding here is IEEE (no fast-math, no reciprocal approximation): the codes
+// and scales must match the CPU definition bit for bit.
+#include "common.h"
+#include "numeric.h"
+
+namespace qmm {
+namespace {
+
+constexpr int64_t kCounterBytes = 64 << 10;  // start of the workspace: split-K counters, kept at zero
+
+__global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v) {
+    int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// amax over the middle axis of [outer, R, inner] when inner > 1 (strided reduction).
+// grid (ceil(inner/64), outer, row_splits); 256 threads = 4 row lanes x 64 columns.
+template <int DT>
+__global__ __launch_bounds__(256) void amax_strided_kernel(const void *__restrict__ w, uint32_t *__restrict__ amax_bits,
+                                                           int64_t R, int64_t inner, int64_t rows_per_split,
+                                                           int use_atomic) {
+    __shared__ float red[4][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t col = int64_t(blockIdx.x) * 64 + tx;
+    const int64_t o = blockIdx.y;
+    const int64_t r0 = int64_t(blockIdx.z) * rows_per_split;
+    const int64_t r1 = min(R, r0 + rows_per_split);
+    float m = 0.0f;
+    if (col < inner) {
+        const int64_t base = o * R * inner + col;
+        int64_t r = r0 + ty;
+        for (; r + 28 < r1; r += 32) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = load_as_f32<DT>(w, base + (r + 4 * i) * inner);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) m = fmaxf(m, fabsf(v[i]));
+        }
+        for (; r < r1; r += 4) m = fmaxf(m, fabsf(load_as_f32<DT>(w, base + r * inner)));
+    }
+    red[ty][tx] = m;
+    __syncthreads();
+    if (ty == 0 && col < inner) {
+        m = fmaxf(fmaxf(red[0][tx], red[1][tx]), fmaxf(red[2][tx], red[3][tx]));
+        // |x| >= 0: the unsigned order of the bit patterns is the order of the values
+        if (use_atomic) atomicMax(&amax_bits[o * inner + col], __float_as_uint(m));
+        else amax_bits[o * inner + col] = __float_as_uint(m);
+    }
+}
+
+// amax over the last axis of [outer, R] (inner == 1): one wave per row, 4 rows per block.
+template <int DT>
+__global__ __launch_bounds__(256) void amax_contig_kernel(const void *__restrict__ w, uint32_t *__restrict__ amax_bits,
+                                                          int64_t outer, int64_t R) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = int64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (row >= outer) return;
+    float m = 0.0f;
+    for (int64_t r = lane; r < R; r += 64) m = fmaxf(m, fabsf(load_as_f32<DT>(w, row * R + r)));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if (lane == 0) amax_bits[row] = __float_as_uint(m);
+}
+
+template <int QT>
+__device__ __forceinline__ void store_code(void *q, int64_t i, float r) {
+    if (QT == HIDET_QMM_I8) {
+        static_cast<int8_t *>(q)[i] = static_cast<int8_t>(fminf(fmaxf(r, -128.0f), 127.0f));
+    } else {
+        static_cast<int16_t *>(q)[i] = static_cast<int16_t>(fminf(fmaxf(r, -32768.0f), 32767.0f));
+    }
+}
+
+// code = saturating_cast(round_half_away(rnd(w / scale))), scale = rnd(amax / qmax), rnd = round to w's dtype.
+template <int DT, int QT>
+__global__ __launch_bounds__(256) void quantize_kernel(const void *__restrict__ w, const uint32_t *__restrict__ amax_bits,
+                                                       void *__restrict__ q, void *__restrict__ scale, int64_t R,
+                                                       int64_t inner, int64_t total) {
+    const float qmax = QT == HIDET_QMM_I8 ? 127.0f : 32767.0f;
+    int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int64_t o = i / (R * inner);
+    const int64_t rem = i - o * R * inner;
+    const int64_t r = rem / inner, c = rem - r * inner;
+    const float amax = __uint_as_float(amax_bits[o * inner + c]);
+    const float s = round_to<DT>(amax / qmax);
+    if (r == 0) store_from_f32<DT>(scale, o * inner + c, s);
+    float code = 0.0f;
+    if (s != 0.0f) code = roundf(round_to<DT>(load_as_f32<DT>(w, i) / s));
+    store_code<QT>(q, i, code);
+}
+
+template <int QT, int ST>
+__global__ __launch_bounds__(256) void dequantize_kernel(const void *__restrict__ q, const void *__restrict__ scale,
+                                                         void *__restrict__ w, int64_t R, int64_t inner, int64_t total) {
+    int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int64_t o = i / (R * inner);
+    const int64_t c = (i - o * R * inner) % inner;
+    const float code = QT == HIDET_QMM_I8 ? float(static_cast<const int8_t *>(q)[i]) : float(static_cast<const int16_t *>(q)[i]);
+    store_from_f32<ST>(w, i, round_to<ST>(code * load_as_f32<ST>(scale, o * inner + c)));
+}
+
+// Group-wise int4: grid (ceil(n/128), k/group); 256 threads = 4 row lanes x 64 column pairs.
+// scale32 = amax / 7 and code = clamp(round_half_away(w / scale32), -7, 7) in float32; two codes per
+// byte along n, low nibble first; the stored scale is scale32 rounded to the scale dtype.
+template <int ST>
+__global__ __launch_bounds__(256) void group_quantize_int4_kernel(const float *__restrict__ w, uint8_t *__restrict__ packed,
+                                                                  void *__restrict__ scales, int64_t n, int group) {
+    __shared__ float red[4][128];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t c0 = int64_t(blockIdx.x) * 128 + 2 * tx;
+    const int64_t g = blockIdx.y;
+    const int64_t rbase = g * group;
+    const bool ok = c0 < n;  // n is even: the pair is in or out together
+    float m0 = 0.0f, m1 = 0.0f;
+    if (ok) {
+        for (int r = ty; r < group; r += 4) {
+            float2 v = *reinterpret_cast<const float2 *>(w + (rbase + r) * n + c0);
+            m0 = fmaxf(m0, fabsf(v.x));
+            m1 = fmaxf(m1, fabsf(v.y));
+        }
+    }
+    red[ty][2 * tx] = m0;
+    red[ty][2 * tx + 1] = m1;
+    __syncthreads();
+    if (!ok) return;
+    m0 = fmaxf(fmaxf(red[0][2 * tx], red[1][2 * tx]), fmaxf(red[2][2 * tx], red[3][2 * tx]));
+    m1 = fmaxf(fmaxf(red[0][2 * tx + 1], red[1][2 * tx + 1]), fmaxf(red[2][2 * tx + 1], red[3][2 * tx + 1]));
+    const float s0 = m0 / 7.0f, s1 = m1 / 7.0f;
+    if (ty == 0) {
+        store_from_f32<ST>(scales, g * n + c0, round_to<ST>(s0));
+        store_from_f32<ST>(scales, g * n + c0 + 1, round_to<ST>(s1));
+    }
+    for (int r = ty; r < group; r += 4) {
+        float2 v = *reinterpret_cast<const float2 *>(w + (rbase + r) * n + c0);
+        float q0 = s0 == 0.0f ? 0.0f : fminf(fmaxf(roundf(v.x / s0), -7.0f), 7.0f);
+        float q1 = s1 == 0.0f ? 0.0f : fminf(fmaxf(roundf(v.y / s1), -7.0f), 7.0f);
+        packed[((rbase + r) * n + c0) >> 1] = uint8_t((int(q0) & 0xF) | ((int(q1) & 0xF) << 4));
+    }
+}
+
+// ---- per-tensor float8 e4m3 -------------------------------------------------------------------
+
+template <int DT>
+__global__ __launch_bounds__(256) void amax_all_kernel(const void *__restrict__ x, uint32_t *__restrict__ amax_bits, int64_t numel) {
+    __shared__ float red[4];
+    float m = 0.0f;
+    for (int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x; i < numel; i += int64_t(gridDim.x) * 256)
+        m = fmaxf(m, fabsf(load_as_f32<DT>(x, i)));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        atomicMax(amax_bits, __float_as_uint(m));
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void fp8_quantize_kernel(const void *__restrict__ x, const uint32_t *__restrict__ amax_bits,
+                                                           uint8_t *__restrict__ codes, float *__restrict__ scale, int64_t numel) {
+    const float s = __uint_as_float(*amax_bits) / 448.0f;
+    int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i == 0) *scale = s;
+    if (i >= numel) return;
+    codes[i] = s == 0.0f ? uint8_t(0) : f32_to_e4m3(load_as_f32<DT>(x, i) / s);
+}
+
+template <typename F>
+void dispatch_float(int dt, F &&f) {
+    switch (dt) {
+        case HIDET_QMM_F32: f(std::integral_constant<int, HIDET_QMM_F32>()); break;
+        case HIDET_QMM_F16: f(std::integral_constant<int, HIDET_QMM_F16>()); break;
+        case HIDET_QMM_BF16: f(std::integral_constant<int, HIDET_QMM_BF16>()); break;
+        default: QMM_FAIL("expected a float32, float16 or bfloat16 dtype code, got " << dt);
+    }
+}
+
+}  // namespace
+}  // namespace qmm
+
+using namespace qmm;
+
+HIDET_API void hidet_symmetric_quantize(const void *w, void *wq, void *scale, int64_t outer, int64_t reduce,
+                                        int64_t inner, int w_dtype, int q_dtype, void *workspace,
+                                        int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(q_dtype == HIDET_QMM_I8 || q_dtype == HIDET_QMM_I16, "quant_type must be int8 or int16, got code " << q_dtype);
+    QMM_CHECK(outer >= 0 && reduce >= 0 && inner >= 0, "negative extent");
+    const int64_t total = outer * reduce * inner;
+    const int64_t nscale = outer * inner;
+    if (nscale == 0) return;
+    QMM_CHECK(w && wq && scale, "null tensor pointer");
+    QMM_CHECK(inner < (int64_t(1) << 31) * 64 && outer < 65536 * int64_t(4), "extent too large");
+    QMM_CHECK(workspace && workspace_bytes >= kCounterBytes + nscale * 4,
+              "workspace too small: need " << kCounterBytes + nscale * 4 << " bytes, got " << workspace_bytes);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    uint32_t *amax_bits = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kCounterBytes);
+    dispatch_float(w_dtype, [&](auto dt) {
+        constexpr int DT = decltype(dt)::value;
+        if (reduce == 0) {
+            launch_aux(fill_u32_kernel, dim3(cdiv(nscale, 256)), dim3(256), 0, stream, amax_bits, nscale, 0u);
+        } else if (inner == 1) {
+            launch(amax_contig_kernel<DT>, dim3(cdiv(outer, 4)), dim3(256), 0, stream, w, amax_bits, outer, reduce);
+        } else {
+            QMM_CHECK(outer <= 65535, "outer extent " << outer << " exceeds the grid limit");
+            const int64_t col_blocks = cdiv(inner, 64);
+            int64_t splits = 1;
+            if (col_blocks * outer < 1024) splits = std::min<int64_t>(cdiv(1024, col_blocks * outer), cdiv(reduce, 64));
+            splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
+            const int64_t rows_per_split = cdiv(cdiv(reduce, splits), 4) * 4;
+            splits = cdiv(reduce, rows_per_split);
+            if (splits > 1) launch_aux(fill_u32_kernel, dim3(cdiv(nscale, 256)), dim3(256), 0, stream, amax_bits, nscale, 0u);
+            launch(amax_strided_kernel<DT>, dim3(col_blocks, outer, splits), dim3(256), 0, stream, w, amax_bits, reduce,
+                   inner, rows_per_split, int(splits > 1));
+        }
+        if (total == 0) return;
+        if (q_dtype == HIDET_QMM_I8)
+            launch(quantize_kernel<DT, HIDET_QMM_I8>, dim3(cdiv(total, 256)), dim3(256), 0, stream, w, amax_bits, wq, scale,
+                   reduce, inner, total);
+        else
+            launch(quantize_kernel<DT, HIDET_QMM_I16>, dim3(cdiv(total, 256)), dim3(256), 0, stream, w, amax_bits, wq, scale,
+                   reduce, inner, total);
+    });
+    if (reduce == 0) {
+        // no elements: scale = 0 still has to be written
+        dispatch_float(w_dtype, [&](auto dt) {
+            constexpr int DT = decltype(dt)::value;
+            if (DT == HIDET_QMM_F32) launch_aux(fill_u32_kernel, dim3(cdiv(nscale, 256)), dim3(256), 0, stream, static_cast<uint32_t *>(scale), nscale, 0u);
+            else launch_aux(fill_u32_kernel, dim3(cdiv(cdiv(nscale, 2), 256)), dim3(256), 0, stream, static_cast<uint32_t *>(scale), cdiv(nscale, 2), 0u);
+        });
+    }
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_symmetric_dequantize(const void *wq, const void *scale, void *w, int64_t outer, int64_t reduce,
+                                          int64_t inner, int q_dtype, int s_dtype, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(q_dtype == HIDET_QMM_I8 || q_dtype == HIDET_QMM_I16, "quantized dtype must be int8 or int16, got code " << q_dtype);
+    const int64_t total = outer * reduce * inner;
+    if (total == 0) return;
+    QMM_CHECK(w && wq && scale, "null tensor pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    dispatch_float(s_dtype, [&](auto dt) {
+        constexpr int ST = decltype(dt)::value;
+        if (q_dtype == HIDET_QMM_I8)
+            launch(dequantize_kernel<HIDET_QMM_I8, ST>, dim3(cdiv(total, 256)), dim3(256), 0, stream, wq, scale, w, reduce, inner, total);
+        else
+            launch(dequantize_kernel<HIDET_QMM_I16, ST>, dim3(cdiv(total, 256)), dim3(256), 0, stream, wq, scale, w, reduce, inner, total);
+    });
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_group_quantize_int4(const void *w, void *packed, void *scales, int64_t k, int64_t n, int group_size,
+                                         int w_dtype, int s_dtype, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(w_dtype == HIDET_QMM_F32, "group_quantize_int4 expects float32 weights, got dtype code " << w_dtype);
+    QMM_CHECK(group_size > 0 && k % group_size == 0, "K (" << k << ") must be a multiple of the group size (" << group_size << ")");
+    QMM_CHECK(n % 2 == 0, "N (" << n << ") must be even: two codes are packed per byte");
+    if (k == 0 || n == 0) return;
+    QMM_CHECK(w && packed && scales, "null tensor pointer");
+    QMM_CHECK(aligned(w, 8), "weight pointer must be 8-byte aligned");
+    QMM_CHECK(k / group_size <= 65535, "too many groups");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    dispatch_float(s_dtype, [&](auto dt) {
+        constexpr int ST = decltype(dt)::value;
+        launch(group_quantize_int4_kernel<ST>, dim3(cdiv(n, 128), k / group_size), dim3(256), 0, stream,
+               static_cast<const float *>(w), static_cast<uint8_t *>(packed), scales, n, group_size);
+    });
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *scale, int64_t numel, int x_dtype,
+                                             void *workspace, int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(scale, "null scale pointer");
+    QMM_CHECK(workspace && workspace_bytes >= kCounterBytes + 4, "workspace too small");
+    QMM_CHECK(numel == 0 || (x && codes), "null tensor pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    uint32_t *amax_bits = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kCounterBytes);
+    launch_aux(fill_u32_kernel, dim3(1), dim3(64), 0, stream, amax_bits, int64_t(1), 0u);
+    dispatch_float(x_dtype, [&](auto dt) {
+        constexpr int DT = decltype(dt)::value;
+        if (numel > 0) {
+            const int64_t blocks = std::min<int64_t>(cdiv(numel, 256 * 8), 2048);
+            launch(amax_all_kernel<DT>, dim3(blocks), dim3(256), 0, stream, x, amax_bits, numel);
+        }
+        launch(fp8_quantize_kernel<DT>, dim3(std::max<int64_t>(1, cdiv(numel, 256))), dim3(256), 0, stream, x, amax_bits,
+               static_cast<uint8_t *>(codes), static_cast<float *>(scale), numel);
+    });
+    QMM_ENTRY_END
+}

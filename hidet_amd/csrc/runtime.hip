@@ -1,0 +1,80 @@
+// Error state, library facts and the timing hook of libhidet_qmm.so.
+#include "common.h"
+
+namespace {
+struct ErrorState {
+    bool has_error = false;
+    std::string msg;
+};
+ErrorState &error_state() {
+    static thread_local ErrorState s;
+    return s;
+}
+}  // namespace
+
+namespace qmm {
+TimingSlot &timing_slot() {
+    static thread_local TimingSlot s;
+    return s;
+}
+}  // namespace qmm
+
+// Thread-local, read-once error string: the convention of src/hidet/runtime/logging.cpp:14-36.
+HIDET_API void hidet_set_last_error(const char *msg) {
+    ErrorState &s = error_state();
+    if (s.has_error) fprintf(stderr, "Warning: hidet error state has been overridden: %s\n", s.msg.c_str());
+    s.has_error = true;
+    s.msg = msg ? msg : "";
+}
+
+HIDET_API const char *hidet_get_last_error(void) {
+    ErrorState &s = error_state();
+    if (!s.has_error) return nullptr;
+    s.has_error = false;
+    return s.msg.c_str();
+}
+
+HIDET_API int hidet_qmm_abi_version(void) { return HIDET_QMM_ABI_VERSION; }
+HIDET_API const char *hidet_qmm_arch(void) { return "gfx950"; }
+HIDET_API int64_t hidet_qmm_min_workspace_bytes(void) { return int64_t(64) << 20; }
+
+HIDET_API void *hidet_qmm_event_create(void) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        hidet_set_last_error("hipEventCreate failed");
+        return nullptr;
+    }
+    return e;
+}
+
+HIDET_API void hidet_qmm_event_destroy(void *event) {
+    if (event) (void)hipEventDestroy(static_cast<hipEvent_t>(event));
+}
+
+HIDET_API void hidet_qmm_event_record(void *event, void *stream) {
+    QMM_ENTRY_BEGIN
+    QMM_HIP(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_qmm_event_synchronize(void *event) {
+    QMM_ENTRY_BEGIN
+    QMM_HIP(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    QMM_ENTRY_END
+}
+
+HIDET_API float hidet_qmm_event_elapsed_ms(void *start, void *stop) {
+    float ms = -1.0f;
+    hipError_t e = hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop));
+    if (e != hipSuccess) {
+        hidet_set_last_error(hipGetErrorString(e));
+        return -1.0f;
+    }
+    return ms;
+}
+
+HIDET_API void hidet_qmm_arm_timing(void *start_event, void *stop_event) {
+    qmm::TimingSlot &ts = qmm::timing_slot();
+    ts.start = static_cast<hipEvent_t>(start_event);
+    ts.stop = static_cast<hipEvent_t>(stop_event);
+}

@@ -1,0 +1,129 @@
+"""ctypes boundary to libhidet_qmm.so.
+
+Mirrors how the reference calls a compiled task library: convert arguments to raw pointers and fixed-width
+integers (python/hidet/ffi/convert.py:56-89), make the ctypes call, then poll `hidet_get_last_error` and raise
+`BackendException` naming the function, its arguments and the library (python/hidet/runtime/compiled_module.py:56-104,
+python/hidet/ffi/ffi.py:46-60).  There is no CPU fallback: if the library is missing or the tensors are not on
+a GPU the call fails.
+"""
+import ctypes
+import os
+from typing import Dict, Optional, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, 'lib', 'libhidet_qmm.so')
+
+_vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+
+# dtype codes of include/hidet_qmm.h
+F32, F16, BF16, I8, I16, E4M3 = 0, 1, 2, 3, 4, 5
+DTYPE_CODE = {
+    torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8, torch.int16: I16,
+    torch.float8_e4m3fn: E4M3,
+}
+
+# name -> (restype, argtypes): every symbol include/hidet_qmm.h declares
+SIGNATURES = {
+    'hidet_set_last_error': (None, [ctypes.c_char_p]),
+    'hidet_get_last_error': (ctypes.c_char_p, []),
+    'hidet_qmm_abi_version': (_i32, []),
+    'hidet_qmm_arch': (ctypes.c_char_p, []),
+    'hidet_qmm_min_workspace_bytes': (_i64, []),
+    'hidet_qmm_event_create': (_vp, []),
+    'hidet_qmm_event_destroy': (None, [_vp]),
+    'hidet_qmm_event_record': (None, [_vp, _vp]),
+    'hidet_qmm_event_synchronize': (None, [_vp]),
+    'hidet_qmm_event_elapsed_ms': (_f32, [_vp, _vp]),
+    'hidet_qmm_arm_timing': (None, [_vp, _vp]),
+    'hidet_symmetric_quantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _i64, _vp]),
+    'hidet_symmetric_dequantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
+    'hidet_symmetric_quant_matmul_f16_i8': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
+}
+
+
+class BackendException(Exception):
+    """Raised when an entry point reported an error (same name as hidet.ffi.ffi.BackendException)."""
+
+
+_LIB: Optional[ctypes.CDLL] = None
+
+
+def load_library() -> ctypes.CDLL:
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError('{} not found: build it with `python -m hidet_amd.build` (hipcc, gfx950)'.format(LIB_PATH))
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = restype, argtypes
+        if lib.hidet_qmm_abi_version() != 1:
+            raise OSError('{} has ABI version {}, expected 1'.format(LIB_PATH, lib.hidet_qmm_abi_version()))
+        _LIB = lib
+    return _LIB
+
+
+def get_last_error() -> Optional[str]:
+    ret = load_library().hidet_get_last_error()
+    return ret.decode('utf-8') if isinstance(ret, bytes) else None
+
+
+def _describe(arg) -> str:
+    if isinstance(arg, torch.Tensor):
+        return 'torch.Tensor(shape={}, dtype={}, device={})'.format(tuple(arg.shape), arg.dtype, arg.device)
+    return str(arg)
+
+
+def call(name: str, *args):
+    """Call `name` with torch tensors (passed as data pointers) and Python scalars; raise on a reported error."""
+    lib = load_library()
+    cargs = []
+    for a in args:
+        if isinstance(a, torch.Tensor):
+            if not a.is_cuda:
+                raise BackendException('{}: tensor argument is on {}, the kernels run on the GPU only'.format(name, a.device))
+            cargs.append(a.data_ptr())
+        else:
+            cargs.append(a)
+    ret = getattr(lib, name)(*cargs)
+    status = get_last_error()
+    if status is not None:
+        raise BackendException('Calling {} with arguments ({}) failed. error:\n{}\nFunction @ {}'.format(
+            name, ', '.join(_describe(a) for a in args), status, LIB_PATH))
+    return ret
+
+
+def require_gpu(*tensors: torch.Tensor):
+    """Every operand must live on one GPU; there is no CPU path."""
+    dev = None
+    for t in tensors:
+        if not t.is_cuda:
+            raise BackendException('tensor operand is on {}: the quantized-matmul kernels run on the GPU only '
+                                   '(no CPU fallback)'.format(t.device))
+        if dev is not None and t.device != dev:
+            raise BackendException('operands are on different devices: {} and {}'.format(dev, t.device))
+        dev = t.device
+
+
+def current_stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+_WORKSPACES: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def workspace(device: torch.device, nbytes: int = 0) -> torch.Tensor:
+    """Zero-initialised scratch buffer for (device, current stream); grows, never shrinks.
+
+    Stands in for the reference's grow-only request_hip_workspace (src/hidet/runtime/hip/context.cpp:43-57).
+    One buffer per stream, because two calls that overlap in time must not share it.
+    """
+    need = max(int(nbytes), int(load_library().hidet_qmm_min_workspace_bytes()))
+    key = (device.index if device.index is not None else torch.cuda.current_device(), current_stream(device))
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws

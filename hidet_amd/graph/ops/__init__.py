@@ -1,0 +1,2 @@
+from . import quant
+from .quant import symmetric_quantize, symmetric_dequantize  # python/hidet/graph/ops/__init__.py:40

@@ -1,0 +1,75 @@
+"""symmetric_quant_matmul with the reference's signature, checks and error texts
+(python/hidet/graph/ops/quant/matmul.py:24-93), executed by `hidet_symmetric_quant_matmul_f16_i8`."""
+from typing import List
+
+import torch
+
+from hidet_amd import ffi, option
+from hidet_amd.graph.operator import Operator, Task, TensorSpec, input_like
+
+
+def _check_task_operands(task: Task, a: TensorSpec, weight: TensorSpec, scale: TensorSpec):
+    task._assert(a.dtype == 'float16' and weight.dtype == 'int8', 'Expect a to be float16 and weight to be int8')
+    if len(a.shape) < 2 or len(weight.shape) != 2:
+        raise ValueError('SymmetricQuantizedMatmul expect , got {} and {}'.format(list(a.shape), list(weight.shape)))
+    task._assert(len(scale.shape) >= 1 and scale.shape[0] == weight.shape[1])
+    task._assert(
+        a.shape[-1] == weight.shape[-2],
+        'Matrix multiplication expect tensor A and B with shape [..., M, K] and [..., K, N]'
+        ', got {} and {}'.format(list(a.shape), list(weight.shape)),
+    )
+
+
+def check_matmul_args(a: torch.Tensor, weight: torch.Tensor):
+    """The argument checks shared by every W8A16 entry (python/hidet/graph/ops/quant/matmul.py:83-92)."""
+    if len(a.shape) < 2 or len(weight.shape) < 2:
+        raise ValueError('a and b must have at least 2 dimensions, got shape {} and {}'.format(list(a.shape), list(weight.shape)))
+    if a.shape[-1] % 2 != 0 or weight.shape[-1] % 2 != 0:
+        raise ValueError('Expect the last dimension of the input tensors to be a multiple of 2')
+    if a.dtype != torch.float16 or weight.dtype != torch.int8:
+        raise ValueError('BatchMatmulF16Op only support float16, int8, got {} and {}'.format(a.dtype, weight.dtype))
+
+
+class SymmetricQuantizedMatmulTask(Task):
+    def __init__(self, a: TensorSpec, weight: TensorSpec, scale: TensorSpec):
+        _check_task_operands(self, a, weight, scale)
+        c_shape = tuple(a.shape[:-1]) + (weight.shape[-1],)
+        super().__init__(name='symmetric_quantized_matmul', inputs=[a, weight, scale],
+                         outputs=[TensorSpec('c', 'float16', c_shape)], attrs={})
+
+
+def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parallel_k_parts: int = 0) -> torch.Tensor:
+    """c[..., M, N] on the GPU.  Leading axes of `a` are folded into M: the weight is 2-D, so broadcasting
+    over them is the same as one tall matmul."""
+    ffi.require_gpu(a, weight, scale)
+    k, n = weight.shape
+    a2 = a.reshape(-1, k)
+    if a2.stride(-1) != 1 or (a2.shape[0] > 1 and a2.stride(0) < k):
+        a2 = a2.contiguous()
+    m = a2.shape[0]
+    lda = a2.stride(0) if m > 1 else k
+    weight = weight.contiguous()
+    scale = scale.contiguous()
+    c = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    ws = ffi.workspace(a.device)
+    ffi.call('hidet_symmetric_quant_matmul_f16_i8', a2, weight, scale, c, m, k, n, lda, int(parallel_k_parts), ws,
+             ws.numel(), ffi.current_stream(a.device))
+    return c.reshape(tuple(a.shape[:-1]) + (n,))
+
+
+class SymmetricQuantizedMatmulOp(Operator):
+    def __init__(self, a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor):
+        task = SymmetricQuantizedMatmulTask(input_like(a, 'a'), input_like(b, 'b'), input_like(scale, 'scale'))
+        super().__init__(inputs=[a, b, scale], attributes={}, task=task)
+
+    def run(self) -> List[torch.Tensor]:
+        from .resolve import resolve_parallel_k_parts
+
+        a, b, scale = self.inputs
+        parts = resolve_parallel_k_parts(option.get_parallel_k(), a, b)
+        return [run_w8a16(a, b, scale, parts)]
+
+
+def symmetric_quant_matmul(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    check_matmul_args(a, weight)
+    return SymmetricQuantizedMatmulOp(a, weight, scale).outputs[0]

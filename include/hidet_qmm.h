@@ -1,0 +1,93 @@
+/*
+ * C ABI of libhidet_qmm.so: MI355X (gfx950) kernels for Hidet's quantized-matmul operator path.
+ *
+ * Conventions (the ones Hidet's runtime applies to every compiled task library):
+ *   - every symbol is extern "C", default visibility, prefixed `hidet_`
+ *     (reference: include/hidet/runtime/common.h:16-18, python/hidet/backend/codegen.py:60-70);
+ *   - entry points return void; a failure is reported through the thread-local, read-once
+ *     last-error string, which the caller polls after every call
+ *     (reference: python/hidet/backend/codegen.py:72-93, python/hidet/runtime/compiled_module.py:79-102);
+ *   - arguments are inputs first, then outputs, as raw device pointers, followed by explicit
+ *     extents; the caller owns every buffer, outputs included, and keeps it alive until the stream
+ *     has run the work (reference: python/hidet/runtime/compiled_task.py:146-207);
+ *   - work is enqueued asynchronously on the hipStream_t passed as the last argument (the
+ *     reference keeps one process-global stream, src/hidet/runtime/hip/context.cpp:35-41; here it
+ *     is explicit per call, so there is no global state besides the error string);
+ *   - scratch memory comes from the caller as (workspace, workspace_bytes) instead of the
+ *     reference's grow-only global request_hip_workspace (src/hidet/runtime/hip/context.cpp:43-57).
+ *     The workspace must be zero-filled once when it is allocated; the kernels leave every counter
+ *     they use at zero again.  Two calls that overlap in time (different streams) must not share
+ *     a workspace.
+ *
+ * All tensors are dense row-major.  No function allocates device memory or synchronises.
+ */
+#ifndef HIDET_QMM_H
+#define HIDET_QMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIDET_QMM_ABI_VERSION 1
+
+/* element type codes */
+enum {
+    HIDET_QMM_F32 = 0,
+    HIDET_QMM_F16 = 1,
+    HIDET_QMM_BF16 = 2,
+    HIDET_QMM_I8 = 3,
+    HIDET_QMM_I16 = 4,
+    HIDET_QMM_E4M3 = 5 /* OCP float8 e4m3fn: max 448, no infinities */
+};
+
+/* ---- error state: same two symbols, same semantics as the reference runtime ------------------
+ * replaces include/hidet/runtime/logging.h:60-63 and src/hidet/runtime/logging.cpp:20-36.
+ * hidet_get_last_error returns the message once and clears it; NULL when there is none. */
+void hidet_set_last_error(const char *msg);
+const char *hidet_get_last_error(void);
+
+/* ---- library facts ---------------------------------------------------------------------------*/
+int hidet_qmm_abi_version(void);
+const char *hidet_qmm_arch(void);            /* "gfx950" */
+int64_t hidet_qmm_min_workspace_bytes(void); /* a workspace of this size serves every entry point */
+
+/* ---- timing hook (measurement only) ----------------------------------------------------------
+ * hidet_qmm_arm_timing makes the NEXT compute-kernel launch issued from this thread record its
+ * own begin and end into the two events (the dispatch's timestamps, without launch gaps).  The
+ * role of the reference's CompiledFunction.profile (python/hidet/runtime/compiled_module.py:106-147). */
+void *hidet_qmm_event_create(void);
+void hidet_qmm_event_destroy(void *event);
+void hidet_qmm_event_record(void *event, void *stream);
+void hidet_qmm_event_synchronize(void *event);
+float hidet_qmm_event_elapsed_ms(void *start, void *stop);
+void hidet_qmm_arm_timing(void *start_event, void *stop_event);
+
+/* ---- symmetric quantize / dequantize ---------------------------------------------------------
+ * replaces the auto-scheduled kernels of SymmetricQuantizationTask / SymmetricDeQuantizationTask
+ * (python/hidet/graph/ops/quant/symmetric.py:23-61).  The tensor is viewed as [outer, reduce, inner]
+ * with the reduced axes folded into `reduce`; scale is [outer, inner] in w's dtype.
+ *   scale = max|w| / qmax, wq = saturating_cast(round_half_away(w / scale)), evaluated in w's dtype
+ *   (float32, float16 or bfloat16); a slice of zeros gives scale 0 and codes 0.
+ * q_dtype is HIDET_QMM_I8 or HIDET_QMM_I16. */
+void hidet_symmetric_quantize(const void *w, void *wq, void *scale, int64_t outer, int64_t reduce, int64_t inner,
+                              int w_dtype, int q_dtype, void *workspace, int64_t workspace_bytes, void *stream);
+/* w = cast(wq, scale dtype) * scale */
+void hidet_symmetric_dequantize(const void *wq, const void *scale, void *w, int64_t outer, int64_t reduce,
+                                int64_t inner, int q_dtype, int s_dtype, void *stream);
+
+/* ---- W8A16: c[m, n] = sum_k a[m, k] * (f16(w[k, n]) * scale[n]) --------------------------------
+ * replaces SymmetricQuantizedMatmulTask (python/hidet/graph/ops/quant/matmul.py:24-74) and the
+ * tuned CUDA template SymmetricQuantizedMatmulF16I8Task with its split-K sum
+ * (python/hidet/graph/ops/quant/matmul_f16_i8.py:30-93, resolve.py:99).
+ * a: float16 [m, k] with row stride lda (elements); w: int8 [k, n]; scale: float16 [n]; c: float16 [m, n].
+ * fp32 accumulation.  parallel_k_parts: 0 lets the library choose the K split, > 0 is a hint. */
+void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
+                                         int64_t k, int64_t n, int64_t lda, int parallel_k_parts, void *workspace,
+                                         int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIDET_QMM_H */

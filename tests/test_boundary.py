@@ -1,0 +1,119 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports every symbol the header
+declares, the error convention works (the reference's tests/runtime/test_try_catch.py), the Python operator
+mirror validates arguments with the reference's messages, and nothing falls back to a CPU path."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import hidet_amd
+from hidet_amd import ffi
+from hidet_amd.graph.ops import quant
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, 'include', 'hidet_qmm.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(hidet_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ffi.load_library()
+    names = declared_symbols()
+    assert len(names) >= 14
+    for name in names:
+        assert hasattr(lib, name), name
+        assert name in ffi.SIGNATURES, 'no ctypes signature for ' + name
+    assert sorted(ffi.SIGNATURES) == names
+    assert lib.hidet_qmm_abi_version() == 1
+    assert lib.hidet_qmm_arch() == b'gfx950'
+    assert lib.hidet_qmm_min_workspace_bytes() >= (1 << 20)
+
+
+def test_error_state_is_read_once():
+    lib = ffi.load_library()
+    assert ffi.get_last_error() is None
+    lib.hidet_set_last_error(b'This is a runtime exception.')
+    assert ffi.get_last_error() == 'This is a runtime exception.'
+    assert ffi.get_last_error() is None
+
+
+def test_entry_point_reports_errors_through_last_error():
+    # argument checks run before anything touches the GPU, so this is safe without one
+    lib = ffi.load_library()
+    lib.hidet_symmetric_quant_matmul_f16_i8(None, None, None, None, 4, 8, 8, 4, 0, None, 0, None)  # lda < k
+    msg = ffi.get_last_error()
+    assert msg is not None and 'row stride' in msg
+    lib.hidet_symmetric_quantize(None, None, None, 1, 1, 1, 0, 0, None, 0, None)  # q_dtype f32 is not a code type
+    assert 'int8 or int16' in ffi.get_last_error()
+    lib.hidet_symmetric_quant_matmul_f16_i8(None, None, None, None, 0, 8, 8, 8, 0, None, 0, None)  # empty: no error
+    assert ffi.get_last_error() is None
+
+
+def test_no_cpu_fallback():
+    a = torch.zeros(2, 4, dtype=torch.float16)
+    w = torch.zeros(4, 4, dtype=torch.int8)
+    s = torch.zeros(4, dtype=torch.float16)
+    with pytest.raises(hidet_amd.BackendException, match='GPU only'):
+        quant.symmetric_quant_matmul(a, w, s)
+    with pytest.raises(hidet_amd.BackendException, match='GPU only'):
+        quant.symmetric_quantize(torch.zeros(4, 4))
+    with pytest.raises(hidet_amd.BackendException, match='GPU only'):
+        quant.symmetric_dequantize(w, s, dims=0)
+
+
+def test_argument_validation_matches_reference_messages():
+    f16, i8 = torch.float16, torch.int8
+    with pytest.raises(ValueError, match='at least 2 dimensions'):
+        quant.symmetric_quant_matmul(torch.zeros(4, dtype=f16), torch.zeros(4, 4, dtype=i8), torch.zeros(4, dtype=f16))
+    with pytest.raises(ValueError, match='multiple of 2'):
+        quant.symmetric_quant_matmul(torch.zeros(2, 3, dtype=f16), torch.zeros(3, 4, dtype=i8), torch.zeros(4, dtype=f16))
+    with pytest.raises(ValueError, match='only support float16, int8'):
+        quant.symmetric_quant_matmul(torch.zeros(2, 4), torch.zeros(4, 4, dtype=i8), torch.zeros(4, dtype=f16))
+    with pytest.raises(ValueError, match=r'expect tensor A and B with shape'):
+        quant.symmetric_quant_matmul(torch.zeros(2, 4, dtype=f16), torch.zeros(6, 4, dtype=i8), torch.zeros(4, dtype=f16))
+    with pytest.raises(ValueError):  # scale length must equal N
+        quant.symmetric_quant_matmul(torch.zeros(2, 4, dtype=f16), torch.zeros(4, 4, dtype=i8), torch.zeros(6, dtype=f16))
+    with pytest.raises(ValueError, match='SymmetricQuantizedMatmul expect'):
+        quant.symmetric_quant_matmul(torch.zeros(2, 4, dtype=f16), torch.zeros(1, 4, 4, dtype=i8), torch.zeros(4, dtype=f16))
+    with pytest.raises(ValueError, match='int8 and int16'):
+        quant.symmetric_quantize(torch.zeros(4, 4), 'float16')
+    with pytest.raises(ValueError):
+        quant.symmetric_quantize(torch.zeros(4, 4), 'int8', dims=2)
+
+
+def test_resolve_policy():
+    from hidet_amd.graph.ops.quant import resolve
+    # the reference's formula (python/hidet/graph/ops/quant/resolve.py:42-48) by direct evaluation
+    assert resolve.reference_k_parts('default', 1, 1, 11008, 4096) == 3
+    assert resolve.reference_k_parts('default', 1, 1, 4096, 11008) == 7
+    assert resolve.reference_k_parts('disabled', 1, 1, 4096, 11008) == 1
+    assert resolve.reference_k_parts(40, 1, 1, 1, 1) == 32 and resolve.reference_k_parts(-3, 1, 1, 1, 1) == 1
+    a, b = torch.zeros(1, 64, dtype=torch.float16), torch.zeros(64, 64, dtype=torch.int8)
+    assert resolve.resolve_parallel_k_parts('disabled', a, b) == 0
+    assert resolve.resolve_parallel_k_parts('default', a, b) == 0
+    assert resolve.resolve_parallel_k_parts(99, a, b) == 32
+    with pytest.raises(ValueError, match='invalid parallel_k'):
+        resolve.resolve_parallel_k_parts('bogus', a, b)
+    with pytest.raises(ValueError):
+        hidet_amd.option.parallel_k('bogus')
+    assert hidet_amd.option.get_parallel_k() == 'disabled'  # the reference's default (python/hidet/option.py:366-369)
+
+
+def test_task_descriptions():
+    from hidet_amd.graph.operator import TensorSpec
+    from hidet_amd.graph.ops.quant.matmul import SymmetricQuantizedMatmulTask
+    from hidet_amd.graph.ops.quant.matmul_f16_i8 import SymmetricQuantizedMatmulF16I8Task
+    from hidet_amd.graph.ops.quant.symmetric import SymmetricQuantizationTask
+    a, w, s = TensorSpec('a', 'float16', (2, 16, 32)), TensorSpec('b', 'int8', (32, 64)), TensorSpec('scale', 'float16', (64,))
+    t = SymmetricQuantizedMatmulTask(a, w, s)
+    assert t.name == 'symmetric_quantized_matmul' and t.outputs[0].shape == (2, 16, 64) and t.outputs[0].dtype == 'float16'
+    t = SymmetricQuantizedMatmulF16I8Task(a, w, s, 3)
+    assert t.name == 'symmetric_quantized_matmulf16' and t.outputs[0].shape == (3, 2, 16, 64)
+    assert t.attrs == {'parallel_k_parts': 3} and not t.allow_prologue()
+    t = SymmetricQuantizationTask(TensorSpec('w', 'float32', (32, 64)), torch.int8, dims=0)
+    assert t.name == 'symmetric_quantization' and t.outputs[1].shape == (64,) and t.attrs['dims'] == [0]

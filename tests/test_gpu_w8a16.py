@@ -1,0 +1,135 @@
+"""GPU parity of the W8A16 matmul entry points against the oracle (dequantize, then matmul with fp32
+accumulation): max |out - ref| / max |ref| <= 1e-2, and exact equality on small-integer inputs."""
+import numpy as np
+import pytest
+import torch
+
+import hidet_amd
+from oracle import clib
+from oracle import oracle as O
+from hidet_amd.graph.ops import quant
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2  # max relative error (normalised by max |ref|) for float16 outputs
+
+
+def _case(seed, m, k, n):
+    a32, w32 = O.make_inputs(seed, m, k, n)
+    a = a32.astype(np.float16)
+    q, s32 = O.symmetric_quantize(w32, 'int8', dims=0)
+    return a, q, s32.astype(np.float16)
+
+
+def _int_case(seed, m, k, n):
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-2, 3, (m, k)).astype(np.float16)
+    q = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    s = (2.0 ** rng.integers(-12, -9, n)).astype(np.float16)
+    return a, q, s
+
+
+@pytest.mark.parametrize('m,k,n', [(1, 256, 256), (1, 4096, 512), (3, 1024, 768), (16, 512, 256), (7, 96, 48),
+                                   (1, 40, 16), (2, 8, 16), (1, 4096, 272), (16, 4096, 4096)])
+def test_exact_on_small_integers(m, k, n):
+    # integer activations and codes with power-of-two scales: every product and partial sum is exact in
+    # fp32, so any dropped row, wrong byte or lost K slice shows as a whole-number difference
+    announce('w8a16 exact', m, k, n)
+    a, q, s = _int_case(m * 1000 + n, m, k, n)
+    want = ((a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :])
+    got = host(quant.symmetric_quant_matmul(dev(a), dev(q), dev(s)))
+    assert np.array_equal(got, want.astype(np.float32).astype(np.float16))
+
+
+@pytest.mark.parametrize('x_shape,w_shape', [[[2, 32, 32], [32, 32]], [[1, 64, 64], [64, 128]]])
+def test_reference_recipe(x_shape, w_shape):
+    # tests/operators_core/test_quantization.py:39-47: quantized result vs the UNquantized matmul at 2e-1
+    announce('w8a16 reference recipe', x_shape, w_shape)
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal(x_shape).astype(np.float16)
+    w = rng.standard_normal(w_shape).astype(np.float16)
+    wq, scale = quant.symmetric_quantize(dev(w), dims=0, quant_type='int8')
+    yq = quant.symmetric_quant_matmul_f16_i8(dev(x), wq, scale)
+    assert tuple(yq.shape) == (1,) + tuple(x_shape[:-1]) + (w_shape[1],)
+    y = np.matmul(x.astype(np.float32), w.astype(np.float32))
+    assert np.allclose(y, host(yq.sum(0)).astype(np.float32), atol=2e-1, rtol=2e-1)
+    y2 = quant.symmetric_quant_matmul(dev(x), wq, scale)
+    assert np.allclose(y, host(y2).astype(np.float32), atol=2e-1, rtol=2e-1)
+
+
+@pytest.mark.parametrize('m,k,n,seed', [(16, 4096, 4096, 0), (1, 4096, 11008, 0), (1, 4096, 11008, 1),
+                                        (1, 4096, 11008, 2), (1, 4096, 11008, 3), (1, 11008, 4096, 0),
+                                        (1, 11008, 4096, 3), (5, 1000, 528, 0), (33, 512, 256, 0)])
+def test_parity_with_oracle(m, k, n, seed):
+    announce('w8a16 parity', m, k, n, seed)
+    a, q, s = _case(seed, m, k, n)
+    ref = clib.quant_matmul_f32acc(a, q, s)
+    got = host(quant.symmetric_quant_matmul(dev(a), dev(q), dev(s)))
+    err = O.max_rel_err(got, ref)
+    print('max_rel_err', err)
+    assert err <= TOL
+    assert err <= 2e-3  # in practice only float16 rounding of the output separates the two
+
+
+def test_split_k_parts_api_and_hints():
+    announce('w8a16 split-k api')
+    a, q, s = _int_case(5, 3, 100, 32)
+    a[:] = np.clip(a, -2, 2)
+    q[:] = np.clip(q, -7, 7)
+    ta, tq, ts = dev(a), dev(q), dev(s)
+    full = host(quant.symmetric_quant_matmul(ta, tq, ts)).astype(np.float64)
+    for parts in (1, 2, 3, 7, 128):
+        c = quant.symmetric_quant_matmul_f16_i8(ta, tq, ts, parallel_k_parts=parts)
+        assert tuple(c.shape) == (parts, 3, 32)
+        ref = O.quant_matmul_split_k(a, q, s, parts)
+        assert np.array_equal(host(c), ref), parts
+        assert np.array_equal(host(c).astype(np.float64).sum(0), full)
+    for parts in (1, 4, 32):
+        c = quant.symmetric_quant_matmul_atomic_f16_i8(ta, tq, ts, parallel_k_parts=parts)
+        assert np.array_equal(host(c).astype(np.float64), full)
+    a, q, s = _case(0, 2, 2048, 512)
+    base = quant.symmetric_quant_matmul(dev(a), dev(q), dev(s))
+    for hint in (1, 2, 5, 16):
+        hidet_amd.option.parallel_k(hint)
+        try:
+            c = quant.symmetric_quant_matmul(dev(a), dev(q), dev(s))
+        finally:
+            hidet_amd.option.parallel_k('disabled')
+        assert O.max_rel_err(host(c), host(base)) < 1e-3
+
+
+def test_deterministic_and_counters_reset():
+    announce('w8a16 determinism')
+    a, q, s = _case(1, 4, 4096, 1024)
+    ta, tq, ts = dev(a), dev(q), dev(s)
+    first = quant.symmetric_quant_matmul(ta, tq, ts)
+    for _ in range(5):
+        assert torch.equal(quant.symmetric_quant_matmul(ta, tq, ts), first)
+    ws = hidet_amd.ffi.workspace(ta.device)
+    torch.cuda.synchronize()
+    assert int(ws[: 64 << 10].view(torch.int32).abs().sum()) == 0  # split-K counters are back at zero
+
+
+def test_strided_rows_and_unaligned_shapes():
+    announce('w8a16 strided / unaligned')
+    a, q, s = _case(2, 4, 512, 256)
+    big = torch.zeros(4, 1024, dtype=torch.float16, device='cuda')
+    big[:, 256:768] = dev(a)
+    got = host(quant.symmetric_quant_matmul(big[:, 256:768], dev(q), dev(s)))
+    assert O.max_rel_err(got, clib.quant_matmul_f32acc(a, q, s)) <= 2e-3
+    # K not a multiple of 8 (activation rows cannot be loaded 16 bytes at a time), N not a multiple of 16
+    for (m, k, n) in ((2, 100, 64), (3, 64, 40), (1, 34, 6)):
+        a, q, s = _case(3, m, k, n)
+        got = host(quant.symmetric_quant_matmul(dev(a), dev(q), dev(s)))
+        assert O.max_rel_err(got, clib.quant_matmul_f32acc(a, q, s)) <= 2e-3, (m, k, n)
+
+
+def test_workspace_too_small_is_reported():
+    announce('w8a16 small workspace')
+    a, q, s = _case(0, 1, 4096, 4096)
+    ta, tq, ts = dev(a), dev(q), dev(s)
+    c = torch.empty(1, 4096, dtype=torch.float16, device='cuda')
+    ws = torch.zeros(1024, dtype=torch.uint8, device='cuda')
+    with pytest.raises(hidet_amd.BackendException, match='workspace too small'):
+        hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8', ta, tq, ts, c, 1, 4096, 4096, 4096, 0, ws, ws.numel(),
+                           hidet_amd.ffi.current_stream(ta.device))
