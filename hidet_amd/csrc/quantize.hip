@@ -195,7 +195,7 @@ HIDET_API void hidet_symmetric_quantize(const void *w, void *wq, void *scale, in
     const int64_t total = outer * reduce * inner;
     const int64_t nscale = outer * inner;
     if (nscale == 0) return;
-    QMM_CHECK(w && wq && scale, "null tensor pointer");
+    QMM_CHECK(scale && (total == 0 || (w && wq)), "null tensor pointer");
     QMM_CHECK(inner < (int64_t(1) << 31) * 64 && outer < 65536 * int64_t(4), "extent too large");
     QMM_CHECK(workspace && workspace_bytes >= kCounterBytes + nscale * 4,
               "workspace too small: need " << kCounterBytes + nscale * 4 << " bytes, got " << workspace_bytes);

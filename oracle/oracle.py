@@ -137,7 +137,7 @@ def symmetric_quantize(w: np.ndarray, quant_type: str = 'int8', dims: Union[int,
     qmax = np.float32(INT_MAX[quant_type])
     red = _normalize_dims(dims, w.ndim)
     w32 = np.asarray(w, dtype=np.float32)
-    amax = np.max(np.abs(w32), axis=red, keepdims=True)  # exact in any order
+    amax = np.max(np.abs(w32), axis=red, keepdims=True, initial=0)  # exact in any order; empty slice -> 0
     scale32 = _round_to(amax / qmax, dt).astype(np.float32)  # one division, rounded to w's dtype
     with np.errstate(divide='ignore', invalid='ignore'):
         quot = _round_to(w32 / scale32, dt).astype(np.float32)  # one division, rounded to w's dtype
