@@ -140,32 +140,46 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const _Float16 *__res
         return;
     }
 
+    // Cross-workgroup exchange without cache-wide fences: the partial tile is written with agent-scope
+    // (write-through) stores, their completion is awaited, and only then is the arrival counted; the
+    // last workgroup reads the tiles back with agent-scope loads.  A full release/acquire fence would
+    // write back and invalidate the whole L2 once per workgroup, which costs more than the GEMV itself.
     float *mine = partials + (int64_t(tile) * splits + split) * m * kTileN;
     for (int row = 0; row < m; ++row) {
         float v = 0.f;
 #pragma unroll
         for (int wv = 0; wv < kWaves; ++wv) v += red[(wv * m + row) * kRedStride + ridx];
-        mine[row * kTileN + tid] = v;
+        __hip_atomic_store(mine + row * kTileN + tid, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __threadfence();  // publish this workgroup's partial tile device-wide before the arrival count
+    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): every store of this lane has been acknowledged
     __syncthreads();
     if (tid == 0) {
-        const uint32_t old = atomicAdd(&counters[tile], 1u);
+        const uint32_t old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (old == uint32_t(splits - 1));
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();  // acquire: the other workgroups' partial tiles are visible from here on
     if (col < n) {
         const float s = float(scale[col]);
         const float *base = partials + int64_t(tile) * splits * m * kTileN;
         for (int row = 0; row < m; ++row) {
             float v = 0.f;
-            for (int sp = 0; sp < splits; ++sp) v += base[(int64_t(sp) * m + row) * kTileN + tid];
+            for (int sp0 = 0; sp0 < splits; sp0 += 16) {  // 16 loads in flight, added in split order
+                float part[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    part[u] = 0.f;
+                    if (sp0 + u < splits)
+                        part[u] = __hip_atomic_load(base + (int64_t(sp0 + u) * m + row) * kTileN + tid, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) v += part[u];
+            }
             c[int64_t(row) * n + col] = _Float16(v * s);
         }
     }
-    if (tid == 0) atomicExch(&counters[tile], 0u);  // leave the counter at zero for the next call
+    if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
 }
 
 // Any shape the fast kernel cannot take (N not a multiple of 16, misaligned weights): one thread per
@@ -189,6 +203,7 @@ void skinny_w8a16_plan(int64_t k, int64_t n, int hint_parts, int *rows_per_block
     int64_t want = hint_parts > 0 ? hint_parts : std::max<int64_t>(1, (768 + t / 2) / t);
     want = std::min<int64_t>(want, cdiv(k, 128));
     int64_t rpb = cdiv(cdiv(k, want), 128) * 128;
+    if (getenv("QMM_RPB")) rpb = atoi(getenv("QMM_RPB"));
     *rows_per_block = int(rpb);
     *splits = int(cdiv(k, rpb));
     *tiles = int(t);
