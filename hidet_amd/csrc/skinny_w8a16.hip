@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const _Float16 *__res
     if (col < n) {
         const float s = float(scale[col]);
         const float *base = partials + int64_t(tile) * splits * m * kTileN;
-        for (int row = 0; row < m; ++row) {
+        if (m == 1) {
             float v = 0.f;
             for (int sp0 = 0; sp0 < splits; sp0 += 16) {  // 16 loads in flight, added in split order
                 float part[16];
@@ -170,13 +170,36 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const _Float16 *__res
                 for (int u = 0; u < 16; ++u) {
                     part[u] = 0.f;
                     if (sp0 + u < splits)
-                        part[u] = __hip_atomic_load(base + (int64_t(sp0 + u) * m + row) * kTileN + tid, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
+                        part[u] = __hip_atomic_load(base + int64_t(sp0 + u) * kTileN + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
 #pragma unroll
                 for (int u = 0; u < 16; ++u) v += part[u];
             }
-            c[int64_t(row) * n + col] = _Float16(v * s);
+            c[col] = _Float16(v * s);
+        } else {
+            // rows in groups of 4, splits in groups of 4: 16 loads in flight, each row added in split order
+            for (int row0 = 0; row0 < m; row0 += 4) {
+                float v[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int sp0 = 0; sp0 < splits; sp0 += 4) {
+                    float part[4][4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            part[u][r] = 0.f;
+                            if (sp0 + u < splits && row0 + r < m)
+                                part[u][r] = __hip_atomic_load(base + (int64_t(sp0 + u) * m + row0 + r) * kTileN + tid,
+                                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) v[r] += part[u][r];
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (row0 + r < m) c[int64_t(row0 + r) * n + col] = _Float16(v[r] * s);
+            }
         }
     }
     if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
