@@ -158,6 +158,36 @@ def main():
     e1.synchronize()
     hot_us = e0.elapsed_time(e1) / 500 * 1e3
 
+    # ---- second half of the metric: the M = 2048 prefill GEMM of the same weight shape ------------------------
+    MP = 2048
+    gp = torch.Generator(device=device)
+    gp.manual_seed(4321)
+    ap = torch.randn((MP, K), generator=gp, device=device, dtype=torch.float32).to(torch.float16)
+    cp = torch.empty((MP, N), dtype=torch.float16, device=device)
+
+    def launch_prefill(i):
+        ffi.call('hidet_symmetric_quant_matmul_f16_i8', ap, ws[i], ss[i], cp, MP, K, N, K, 0, work, work.numel(), sptr)
+
+    with torch.cuda.stream(stream):
+        for i in range(3):
+            launch_prefill(i)
+    stream.synchronize()
+    rows = np.array([0, 127, 128, 1029, 2047])
+    pref = clib.quant_matmul_f32acc(ap.cpu().numpy()[rows], ws[2].cpu().numpy(), ss[2].cpu().numpy())
+    prefill_parity = O.max_rel_err(cp.cpu().numpy()[rows], pref)
+    ev0, ev1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
+    pd = []
+    for rep in range(24):
+        lib.hidet_qmm_arm_timing(ev0, ev1)
+        launch_prefill(rep % RING)
+        lib.hidet_qmm_event_synchronize(ev1)
+        pd.append(lib.hidet_qmm_event_elapsed_ms(ev0, ev1) * 1e3)
+    lib.hidet_qmm_event_destroy(ev0)
+    lib.hidet_qmm_event_destroy(ev1)
+    pd = np.array(pd[4:])
+    prefill_flops = 2.0 * MP * K * N
+    prefill_tflops = prefill_flops / (pd.mean() * 1e-6) / 1e12
+
     result = {
         'metric': 'w8a16_decode_gemv_bandwidth', 'value': round(value, 1), 'unit': 'GB/s', 'n_gpus': 1,
         'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 5), 'higher_is_better': True,
@@ -172,6 +202,12 @@ def main():
                      'launches_timed': int(durs.size)},
         'llc_hot_single_buffer': {'us_per_launch_back_to_back': round(hot_us, 3),
                                   'GB/s': round(GEMV_BYTES / (hot_us * 1e-6) / 1e9, 1)},
+        'prefill': {'workload': 'W8A16 prefill GEMM, a f16[2048,4096] x w int8[4096,11008] -> f16[2048,11008]',
+                    'value': round(prefill_tflops, 1), 'unit': 'TFLOP/s', 'kernel': 'gemm_w8a16_kernel',
+                    'kernel_us_mean': round(float(pd.mean()), 2), 'kernel_us_min': round(float(pd.min()), 2),
+                    'roofline': {'bound': 'mfma', 'achieved': round(prefill_tflops, 1), 'peak': MFMA_F16_PEAK_TFLOPS,
+                                 'unit': 'TFLOP/s', 'frac': round(prefill_tflops / MFMA_F16_PEAK_TFLOPS, 4)},
+                    'max_rel_err_vs_oracle_rows_sample': prefill_parity},
         'parity': {'max_rel_err_vs_oracle': parity, 'tolerance': 1e-2, 'graph_replay_matches_eager': replay_ok},
     }
     if not args.no_cpu_baseline:

@@ -1,0 +1,39 @@
+// Entry point of the group-wise W4A16 matmul: argument checks and the choice of kernel family.
+#include "common.h"
+
+namespace qmm {
+void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
+                         int64_t lda, int group, int dtype, int parallel_k_parts, void *workspace, int64_t workspace_bytes,
+                         hipStream_t stream);
+bool gemm_w4a16_supported(const void *a, const void *w, const void *scales, const void *c, int64_t k, int64_t n,
+                          int64_t lda, int group);
+void gemm_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
+                       int64_t lda, int group, int dtype, hipStream_t stream);
+}  // namespace qmm
+
+using namespace qmm;
+
+HIDET_API void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, const void *scales, void *c, int64_t m,
+                                                  int64_t k, int64_t n, int64_t lda, int group_size, int dtype,
+                                                  int parallel_k_parts, void *workspace, int64_t workspace_bytes,
+                                                  void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(dtype == HIDET_QMM_BF16 || dtype == HIDET_QMM_F16,
+              "activations and scales must be bfloat16 or float16, got dtype code " << dtype);
+    QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
+    QMM_CHECK(group_size > 0 && k % group_size == 0,
+              "K (" << k << ") must be a multiple of the group size (" << group_size << ")");
+    QMM_CHECK(n % 2 == 0, "N (" << n << ") must be even: two codes are packed per byte");
+    QMM_CHECK(lda >= k, "row stride of a (" << lda << ") is smaller than K (" << k << ")");
+    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    QMM_CHECK(parallel_k_parts >= 0, "parallel_k_parts must be >= 0");
+    if (m == 0 || n == 0) return;
+    QMM_CHECK(a && c && (k == 0 || (w && scales)), "null tensor pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (m > 64 && k > 0 && gemm_w4a16_supported(a, w, scales, c, k, n, lda, group_size))
+        gemm_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, stream);
+    else
+        skinny_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, parallel_k_parts, workspace, workspace_bytes,
+                            stream);
+    QMM_ENTRY_END
+}

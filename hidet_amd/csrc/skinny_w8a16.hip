@@ -11,16 +11,13 @@
 // zero), so M = 1 and M = 16 cost the same.  K is split over the 4 waves of a workgroup (LDS
 // reduction) and over workgroups; the last workgroup to arrive for a column tile adds the partial
 // tiles in a fixed order (deterministic), applies the scale and writes float16.
-#include "common.h"
+#include "skinny_common.h"
 
 namespace qmm {
 namespace {
 
-constexpr int kTileN = 256;
-constexpr int kWaves = 4;
-constexpr int kRedStride = 272;  // 16 lanes x 17 floats: conflict-free LDS writes
-constexpr int64_t kCounterBytes = 64 << 10;
-constexpr int kMaxTiles = int(kCounterBytes / 4);
+constexpr int kTileN = kSkinnyTileN;
+constexpr int kWaves = kSkinnyWaves;
 
 template <int DEPTH, bool ALIGNED_A, bool FOLD>
 __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const _Float16 *__restrict__ a, int64_t lda,
@@ -31,14 +28,8 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const _Float16 *__res
     extern __shared__ float red[];  // [kWaves][m][kRedStride]
     __shared__ int s_last;
 
-    // Workgroups are dealt round-robin to the 8 XCDs: keep every K-split of a column tile on one XCD
-    // so that the partial tiles meet in that XCD's L2.
-    const int bid = blockIdx.x;
-    const int xcd = bid & 7;
-    const int rest = bid >> 3;
-    const int split = rest % splits;
-    const int tile = (rest / splits) * 8 + xcd;
-    if (tile >= tiles) return;
+    int tile, split;
+    if (!skinny_tile_of_block(splits, tiles, &tile, &split)) return;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -113,96 +104,13 @@ __global__ __launch_bounds__(256) void skinny_w8a16_kernel(const _Float16 *__res
         }
     }
 
-    // ---- reduce the 4 waves through LDS; rows 4g + v of the accumulator tile are rows of c ----------
+    if (FOLD) {
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int row = 4 * g + v;
-        if (row < m) {
-            float *dst = red + (wave * m + row) * kRedStride + cl * 17;
+        for (int t = 0; t < 16; ++t)
 #pragma unroll
-            for (int t = 0; t < 16; ++t) dst[t] = FOLD ? acc[t][v] - 1152.0f * xsum[v] : acc[t][v];
-        }
+            for (int v = 0; v < 4; ++v) acc[t][v] -= 1152.0f * xsum[v];
     }
-    __syncthreads();
-
-    const int col = tile * kTileN + tid;
-    const int ridx = tid + (tid >> 4);
-    if (splits == 1) {
-        if (col < n) {
-            const float s = float(scale[col]);
-            for (int row = 0; row < m; ++row) {
-                float v = 0.f;
-#pragma unroll
-                for (int wv = 0; wv < kWaves; ++wv) v += red[(wv * m + row) * kRedStride + ridx];
-                c[int64_t(row) * n + col] = _Float16(v * s);
-            }
-        }
-        return;
-    }
-
-    // Cross-workgroup exchange without cache-wide fences: the partial tile is written with agent-scope
-    // (write-through) stores, their completion is awaited, and only then is the arrival counted; the
-    // last workgroup reads the tiles back with agent-scope loads.  A full release/acquire fence would
-    // write back and invalidate the whole L2 once per workgroup, which costs more than the GEMV itself.
-    float *mine = partials + (int64_t(tile) * splits + split) * m * kTileN;
-    for (int row = 0; row < m; ++row) {
-        float v = 0.f;
-#pragma unroll
-        for (int wv = 0; wv < kWaves; ++wv) v += red[(wv * m + row) * kRedStride + ridx];
-        __hip_atomic_store(mine + row * kTileN + tid, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): every store of this lane has been acknowledged
-    __syncthreads();
-    if (tid == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == uint32_t(splits - 1));
-    }
-    __syncthreads();
-    if (!s_last) return;
-    if (col < n) {
-        const float s = float(scale[col]);
-        const float *base = partials + int64_t(tile) * splits * m * kTileN;
-        if (m == 1) {
-            float v = 0.f;
-            for (int sp0 = 0; sp0 < splits; sp0 += 16) {  // 16 loads in flight, added in split order
-                float part[16];
-#pragma unroll
-                for (int u = 0; u < 16; ++u) {
-                    part[u] = 0.f;
-                    if (sp0 + u < splits)
-                        part[u] = __hip_atomic_load(base + int64_t(sp0 + u) * kTileN + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-#pragma unroll
-                for (int u = 0; u < 16; ++u) v += part[u];
-            }
-            c[col] = _Float16(v * s);
-        } else {
-            // rows in groups of 4, splits in groups of 4: 16 loads in flight, each row added in split order
-            for (int row0 = 0; row0 < m; row0 += 4) {
-                float v[4] = {0.f, 0.f, 0.f, 0.f};
-                for (int sp0 = 0; sp0 < splits; sp0 += 4) {
-                    float part[4][4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            part[u][r] = 0.f;
-                            if (sp0 + u < splits && row0 + r < m)
-                                part[u][r] = __hip_atomic_load(base + (int64_t(sp0 + u) * m + row0 + r) * kTileN + tid,
-                                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        }
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) v[r] += part[u][r];
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (row0 + r < m) c[int64_t(row0 + r) * n + col] = _Float16(v[r] * s);
-            }
-        }
-    }
-    if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
+    skinny_reduce_store<_Float16>(acc, m, n, tile, split, splits, scale, c, partials, counters, red, &s_last);
 }
 
 // Any shape the fast kernel cannot take (N not a multiple of 16, misaligned weights): one thread per
@@ -220,18 +128,6 @@ __global__ __launch_bounds__(256) void naive_w8a16_kernel(const _Float16 *__rest
 
 }  // namespace
 
-// Picks the K split: enough workgroups to keep ~3 per CU in flight, slices of at least 128 rows.
-void skinny_w8a16_plan(int64_t k, int64_t n, int hint_parts, int *rows_per_block, int *splits, int *tiles) {
-    const int64_t t = cdiv(n, kTileN);
-    int64_t want = hint_parts > 0 ? hint_parts : std::max<int64_t>(1, (768 + t / 2) / t);
-    want = std::min<int64_t>(want, cdiv(k, 128));
-    int64_t rpb = cdiv(cdiv(k, want), 128) * 128;
-    if (getenv("QMM_RPB")) rpb = atoi(getenv("QMM_RPB"));
-    *rows_per_block = int(rpb);
-    *splits = int(cdiv(k, rpb));
-    *tiles = int(t);
-}
-
 void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                          int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     const bool fast = (n % 16 == 0) && aligned(w, 16) && k > 0;
@@ -241,8 +137,8 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
         return;
     }
     int rpb, splits, tiles;
-    skinny_w8a16_plan(k, n, parallel_k_parts, &rpb, &splits, &tiles);
-    QMM_CHECK(tiles <= kMaxTiles, "N too large for the split-K counters");
+    skinny_plan(k, n, parallel_k_parts, 128, &rpb, &splits, &tiles);
+    QMM_CHECK(tiles <= kMaxSkinnyTiles, "N too large for the split-K counters");
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16);
     const int grid = int(cdiv(tiles, 8) * 8 * splits);
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
@@ -256,7 +152,7 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
         uint32_t *counters = static_cast<uint32_t *>(workspace);
         const _Float16 *ap = static_cast<const _Float16 *>(a) + m0 * lda;
         _Float16 *cp = static_cast<_Float16 *>(c) + m0 * n;
-        const size_t shmem = size_t(kWaves) * mt * kRedStride * sizeof(float);
+        const size_t shmem = skinny_lds_bytes(mt);
         auto go = [&](auto kern) {
             if (shmem > 65536) QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(shmem)));
             launch(kern, dim3(grid), dim3(256), shmem, stream, ap, lda, static_cast<const int8_t *>(w),

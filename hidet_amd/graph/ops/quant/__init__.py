@@ -4,3 +4,4 @@ from .matmul import symmetric_quant_matmul
 from .matmul_f16_i8 import symmetric_quant_matmul_f16_i8
 from .matmul_f16_i8_atomic import symmetric_quant_matmul_atomic_f16_i8
 from . import resolve
+from .group_int4 import symmetric_group_quantize_int4, symmetric_quant_matmul_w4a16  # group-wise W4A16 (not in the reference)

@@ -87,6 +87,29 @@ void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const voi
                                          int64_t k, int64_t n, int64_t lda, int parallel_k_parts, void *workspace,
                                          int64_t workspace_bytes, void *stream);
 
+/* ---- group-wise W4A16 (benchmark configuration; the reference has no operator for it) -----------
+ * Conventions inherited from the reference: int4b is signed with max 7, so the symmetric rule of
+ * python/hidet/graph/ops/quant/symmetric.py:32-41 gives scale = amax / 7; sub-byte tensors are packed
+ * along the innermost axis, element o in byte o / 2 at bit (o % 2) * 4
+ * (python/hidet/transforms/lower_integer_subbyte.py:103-113), i.e. byte [k, j] = q[k, 2j] | q[k, 2j+1] << 4;
+ * scales are [K / group, N] as in the reference's test kernel (tests/cute_kernel/quantized_linear.py:692-699).
+ *
+ * hidet_group_quantize_int4: w float32 [k, n] -> packed uint8 [k, n/2], scales [k/group, n] (s_dtype:
+ * bfloat16 or float16); scale32 = amax / 7 and code = clamp(round_half_away(w / scale32), -7, 7) in float32. */
+void hidet_group_quantize_int4(const void *w, void *packed, void *scales, int64_t k, int64_t n, int group_size,
+                               int w_dtype, int s_dtype, void *stream);
+/* c[m, n] = sum_g scales[g, n] * sum_{k in g} a[m, k] * q[k, n]; a, scales, c share `dtype` (bfloat16 or
+ * float16); fp32 accumulation. */
+void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k,
+                                        int64_t n, int64_t lda, int group_size, int dtype, int parallel_k_parts,
+                                        void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ---- per-tensor float8 e4m3 quantization (benchmark configuration) --------------------------------
+ * scale[0] = max|x| / 448 (float32, written to device memory), codes = e4m3(x / scale), round to nearest
+ * even, saturating; e4m3 limits from python/hidet/ir/dtypes/floats.py:108-110. */
+void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *scale, int64_t numel, int x_dtype,
+                                   void *workspace, int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

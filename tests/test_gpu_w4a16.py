@@ -1,0 +1,98 @@
+"""GPU parity of group-wise int4 quantization (bit-exact) and the W4A16 matmul (max relative error <= 1e-2
+against the oracle: dequantize to the 16-bit type, then matmul with fp32 accumulation).
+
+The reference has no operator for this configuration: PARITY UNPINNED by reference tests; the oracle is pinned
+by closed forms and the reference's packing convention (tests/test_oracle.py)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from hidet_amd.graph.ops import quant
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _bits16(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize('k,n,g,sdt', [(256, 64, 128, 'bfloat16'), (512, 200, 64, 'float16'), (4096, 11008, 128, 'bfloat16'),
+                                       (128, 2, 32, 'bfloat16')])
+def test_group_quantize_int4_bit_exact(k, n, g, sdt):
+    announce('int4 quantize', k, n, g, sdt)
+    _, w = O.make_inputs(0, 1, k, n)
+    w[0:g, 1] = 0  # an all-zero group: scale 0, codes 0
+    packed, scales = quant.symmetric_group_quantize_int4(dev(w), g, sdt)
+    p0, s0, q0 = O.group_quantize_int4(w, g, sdt)
+    assert np.array_equal(host(packed), p0)
+    want = O.bf16_bits(s0) if sdt == 'bfloat16' else s0.view(np.uint16)
+    assert np.array_equal(_bits16(scales), want)
+    assert np.array_equal(O.unpack_int4(host(packed)), q0)
+
+
+def _case(seed, m, k, n, g, dtype):
+    a32, w = O.make_inputs(seed, m, k, n)
+    packed, scales, q = O.group_quantize_int4(w, g, dtype)
+    if dtype == 'bfloat16':
+        a = O.to_bf16(a32)
+        return a, packed, scales, dev(a, torch.bfloat16), dev(packed), dev(scales, torch.bfloat16)
+    a = a32.astype(np.float16)
+    return a, packed, scales, dev(a), dev(packed), dev(scales)
+
+
+@pytest.mark.parametrize('m,k,n,g', [(1, 256, 256, 128), (3, 512, 768, 128), (16, 4096, 512, 128), (1, 384, 272, 32),
+                                     (7, 128, 48, 64), (2, 96, 6, 32), (1, 4096, 11008, 128), (16, 4096, 11008, 128)])
+@pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
+def test_skinny_parity(m, k, n, g, dtype):
+    announce('w4a16 skinny', m, k, n, g, dtype)
+    a, packed, scales, ta, tp, ts = _case(0, m, k, n, g, dtype)
+    ref = O.w4a16_matmul(a, packed, scales, g, dtype)
+    got = host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g))
+    err = O.max_rel_err(got, ref)
+    print('max_rel_err', err)
+    assert err <= TOL
+    assert err <= (8e-3 if dtype == 'bfloat16' else 2e-3)  # bf16 output rounding is 2^-9 relative
+
+
+@pytest.mark.parametrize('m,k,n,g', [(128, 256, 256, 128), (65, 128, 264, 32), (512, 4096, 1024, 128), (300, 512, 520, 64)])
+@pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
+def test_gemm_parity(m, k, n, g, dtype):
+    announce('w4a16 gemm', m, k, n, g, dtype)
+    a, packed, scales, ta, tp, ts = _case(1, m, k, n, g, dtype)
+    ref = O.w4a16_matmul(a, packed, scales, g, dtype)
+    got = host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g))
+    err = O.max_rel_err(got, ref)
+    print('max_rel_err', err)
+    assert err <= TOL
+    assert err <= (8e-3 if dtype == 'bfloat16' else 2e-3)
+
+
+def test_exact_on_small_integers():
+    announce('w4a16 exact')
+    rng = np.random.default_rng(21)
+    for (m, k, n) in ((4, 256, 256), (128, 256, 128)):
+        a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+        q = rng.integers(-8, 8, (k, n)).astype(np.int8)  # -8 is representable and must decode correctly
+        scales = (2.0 ** rng.integers(-3, 1, (k // 128, n))).astype(np.float32)
+        want = np.zeros((m, n))
+        for g in range(k // 128):
+            want += (a[:, g * 128:(g + 1) * 128].astype(np.int64) @ q[g * 128:(g + 1) * 128].astype(np.int64)) * scales[g]
+        got = host(quant.symmetric_quant_matmul_w4a16(dev(a, torch.bfloat16), dev(O.pack_int4(q)), dev(scales, torch.bfloat16), 128))
+        assert np.array_equal(got, O.to_bf16(want.astype(np.float32))), (m, k, n)
+
+
+def test_full_size_prefill_rows_sample():
+    m, k, n, g = 512, 4096, 11008, 128
+    announce('w4a16 full size', m, k, n)
+    a, packed, scales, ta, tp, ts = _case(0, m, k, n, g, 'bfloat16')
+    got = quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g)
+    rows = np.array([0, 15, 16, 63, 64, 200, 255, 256, 511])
+    ref = O.w4a16_matmul(a[rows], packed, scales, g, 'bfloat16')
+    err = O.max_rel_err(host(got)[rows], ref)
+    print('max_rel_err', err)
+    assert err <= 8e-3
+    skinny = quant.symmetric_quant_matmul_w4a16(ta[torch.from_numpy(rows).cuda()], tp, ts, g)
+    assert O.max_rel_err(host(skinny), host(got)[rows]) <= 8e-3
