@@ -1,0 +1,125 @@
+// FP8 e4m3 decode GEMV / skinny GEMM (M <= 16): c[m, n] = cast(alpha * sum_k a[m, k] * b[n, k]).
+//
+// b is [N, K] with K contiguous, so the reduction runs along the lanes' own loads: lane (kg, ls) of a
+// wave reads 32 consecutive bytes of row n0 + ls at k = kbase + 32 kg; the 16 lanes x 4 k-groups of one
+// k-step cover 16 rows x 128 contiguous bytes.  Those 32 bytes are directly the column operand of
+// the CDNA4 block-scaled MFMA 16x16x128 (unit scales): the matrix core does both the multiply and the
+// cross-lane reduction, and M = 1 costs the same as M = 16.  The 4 waves of a workgroup split K and
+// meet in LDS; a workgroup owns 16 output columns, so N / 16 workgroups stream b exactly once.
+#include "common.h"
+#include "numeric.h"
+
+namespace qmm {
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kDepth = 8;  // k-steps (of 128 bytes) whose loads are issued together
+
+template <int OUT, bool ALIGNED_A>
+__global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda,
+                                                         const uint8_t *__restrict__ b, int64_t ldb, void *__restrict__ c,
+                                                         int m, int n, int k, const float *__restrict__ scale_a,
+                                                         const float *__restrict__ scale_b) {
+    __shared__ float red[kWaves][16][17];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 4, ls = lane & 15;
+    const int n0 = blockIdx.x * 16;
+    const int nrow = n0 + ls;
+    const bool n_ok = nrow < n;
+
+    // K is cut into 128-byte steps dealt to the waves in contiguous runs
+    const int steps = (k + 127) >> 7;
+    const int steps_per_wave = (steps + kWaves - 1) / kWaves;
+    const int s_begin = wave * steps_per_wave, s_end = min(steps, s_begin + steps_per_wave);
+
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t *bp = b + int64_t(nrow) * ldb + 32 * kg;
+    const uint8_t *ap = a + int64_t(ls) * lda + 32 * kg;
+
+    for (int s0 = s_begin; s0 < s_end; s0 += kDepth) {
+        uint4 wv[kDepth][2], xv[kDepth][2];
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            const int kb = (s0 + d) * 128 + 32 * kg;
+            wv[d][0] = wv[d][1] = uint4{0u, 0u, 0u, 0u};
+            if (n_ok && s0 + d < s_end) {
+                if (kb < k) wv[d][0] = *reinterpret_cast<const uint4 *>(bp + int64_t(s0 + d) * 128);
+                if (kb + 16 < k) wv[d][1] = *reinterpret_cast<const uint4 *>(bp + int64_t(s0 + d) * 128 + 16);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            const int kb = (s0 + d) * 128 + 32 * kg;
+            xv[d][0] = xv[d][1] = uint4{0u, 0u, 0u, 0u};
+            if (ls < m && s0 + d < s_end) {
+                if (ALIGNED_A) {
+                    if (kb < k) xv[d][0] = *reinterpret_cast<const uint4 *>(ap + int64_t(s0 + d) * 128);
+                    if (kb + 16 < k) xv[d][1] = *reinterpret_cast<const uint4 *>(ap + int64_t(s0 + d) * 128 + 16);
+                } else {
+                    uint8_t tmp[32];
+#pragma unroll
+                    for (int e = 0; e < 32; ++e) tmp[e] = (kb + e < k) ? ap[int64_t(s0 + d) * 128 + e] : uint8_t(0);
+                    uint32_t wds[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        wds[e] = uint32_t(tmp[4 * e]) | (uint32_t(tmp[4 * e + 1]) << 8) | (uint32_t(tmp[4 * e + 2]) << 16) |
+                                 (uint32_t(tmp[4 * e + 3]) << 24);
+                    xv[d][0] = uint4{wds[0], wds[1], wds[2], wds[3]};
+                    xv[d][1] = uint4{wds[4], wds[5], wds[6], wds[7]};
+                }
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            int8v_t rv, cv;
+            rv[0] = int(xv[d][0].x); rv[1] = int(xv[d][0].y); rv[2] = int(xv[d][0].z); rv[3] = int(xv[d][0].w);
+            rv[4] = int(xv[d][1].x); rv[5] = int(xv[d][1].y); rv[6] = int(xv[d][1].z); rv[7] = int(xv[d][1].w);
+            cv[0] = int(wv[d][0].x); cv[1] = int(wv[d][0].y); cv[2] = int(wv[d][0].z); cv[3] = int(wv[d][0].w);
+            cv[4] = int(wv[d][1].x); cv[5] = int(wv[d][1].y); cv[6] = int(wv[d][1].z); cv[7] = int(wv[d][1].w);
+            // rows = activation rows, columns = rows of b; formats e4m3 x e4m3, unit block scales
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+        }
+    }
+    // acc[v] = partial c[4 kg + v][n0 + ls]
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][4 * kg + v][ls] = acc[v];
+    __syncthreads();
+    const int row = tid >> 4, cn = tid & 15;
+    if (row < m && n0 + cn < n) {
+        float v = red[0][row][cn] + red[1][row][cn] + red[2][row][cn] + red[3][row][cn];
+        if (scale_a != nullptr) v *= *scale_a;
+        if (scale_b != nullptr) v *= *scale_b;
+        const int64_t o = int64_t(row) * n + n0 + cn;
+        if (OUT == HIDET_QMM_F32) static_cast<float *>(c)[o] = v;
+        else if (OUT == HIDET_QMM_BF16) static_cast<uint16_t *>(c)[o] = f32_to_bf16_bits(v);
+        else if (OUT == HIDET_QMM_F16) static_cast<uint16_t *>(c)[o] = f32_to_f16_bits(v);
+        else static_cast<uint8_t *>(c)[o] = f32_to_e4m3(v);
+    }
+}
+
+}  // namespace
+
+bool skinny_fp8_supported(const void *b, int64_t k, int64_t ldb) { return (ldb % 16 == 0) && (k % 16 == 0) && aligned(b, 16) && k > 0; }
+
+void skinny_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                       int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
+    const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
+    const float *sa = static_cast<const float *>(scale_a), *sb = static_cast<const float *>(scale_b);
+    const bool aligned_a = (lda % 16 == 0) && aligned(a, 16);
+    const dim3 grid(uint32_t(cdiv(n, 16)));
+    auto go = [&](auto kern) { launch(kern, grid, dim3(256), 0, stream, ap, lda, bp, ldb, c, int(m), int(n), int(k), sa, sb); };
+#define QMM_FP8_SKINNY(OUT)                                   \
+    if (aligned_a) go(skinny_fp8_kernel<OUT, true>);          \
+    else go(skinny_fp8_kernel<OUT, false>);
+    switch (out_dtype) {
+        case HIDET_QMM_F32: QMM_FP8_SKINNY(HIDET_QMM_F32) break;
+        case HIDET_QMM_F16: QMM_FP8_SKINNY(HIDET_QMM_F16) break;
+        case HIDET_QMM_BF16: QMM_FP8_SKINNY(HIDET_QMM_BF16) break;
+        case HIDET_QMM_E4M3: QMM_FP8_SKINNY(HIDET_QMM_E4M3) break;
+        default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+    }
+#undef QMM_FP8_SKINNY
+}
+
+}  // namespace qmm

@@ -43,6 +43,8 @@ SIGNATURES = {
     'hidet_group_quantize_int4': (None, [_vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
     'hidet_symmetric_quant_matmul_w4a16': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     'hidet_fp8_quantize_per_tensor': (None, [_vp, _vp, _vp, _i64, _i32, _vp, _i64, _vp]),
+    'hidet_matmul_f8': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp]),
+    'hidet_matmul_f8_scaled': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp]),
 }
 
 
@@ -88,6 +90,8 @@ def call(name: str, *args):
             if not a.is_cuda:
                 raise BackendException('{}: tensor argument is on {}, the kernels run on the GPU only'.format(name, a.device))
             cargs.append(a.data_ptr())
+        elif a is None:
+            cargs.append(None)
         else:
             cargs.append(a)
     ret = getattr(lib, name)(*cargs)

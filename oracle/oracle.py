@@ -334,7 +334,7 @@ def e4m3_encode(x: np.ndarray) -> np.ndarray:
 def fp8_quantize_per_tensor(x: np.ndarray) -> Tuple[np.ndarray, np.float32]:
     """scale = amax / 448 (float32), code = e4m3(x / scale)  (benchmark-defined)."""
     x = np.asarray(x, dtype=np.float32)
-    scale = np.float32(np.max(np.abs(x)) / np.float32(448))
+    scale = np.float32(np.max(np.abs(x), initial=0) / np.float32(448))
     if scale == 0:
         return np.zeros(x.shape, dtype=np.uint8), scale
     return e4m3_encode((x / scale).astype(np.float32)), scale

@@ -1,0 +1,150 @@
+"""GPU parity of the FP8 e4m3 path: per-tensor quantization bit-exact against the oracle, matmul_f8 /
+matmul_f8_scaled exact on the reference's integer-valued test recipes
+(tests/operators_core/test_matmul.py:250-373), and max relative error <= 3e-2 on N(0,1) data."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from hidet_amd.graph.ops.matmul import matmul_f8 as F8
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+TOL = 3e-2  # max relative error (normalised by max |ref|) for fp8 matmuls
+
+
+def codes_of(t: torch.Tensor) -> np.ndarray:
+    return t.view(torch.uint8).cpu().numpy()
+
+
+def f8(codes: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(codes)).cuda().view(torch.float8_e4m3fn)
+
+
+def test_quantize_per_tensor_bit_exact():
+    announce('fp8 quantize')
+    rng = np.random.default_rng(3)
+    tab = O.e4m3_decode(np.arange(0, 0x7F, dtype=np.uint8)).astype(np.float64)
+    mids = ((tab[:-1] + tab[1:]) / 2).astype(np.float32)
+    # amax = 448 makes the scale exactly 1, so the codes are e4m3(x): every tie and neighbour of a tie
+    x = np.concatenate([np.array([448.0, -448.0], dtype=np.float32), tab.astype(np.float32), mids, -mids,
+                        np.nextafter(mids, np.float32(1e9)), np.nextafter(mids, np.float32(-1e9)),
+                        rng.uniform(-448, 448, 20000).astype(np.float32),
+                        (rng.standard_normal(20000) * 10.0 ** rng.uniform(-6, 1, 20000)).astype(np.float32)])
+    x = x[np.abs(x) <= 448]
+    codes, scale = F8.fp8_quantize_per_tensor(dev(x))
+    c0, s0 = O.fp8_quantize_per_tensor(x)
+    assert float(scale.item()) == 1.0 == float(s0)
+    assert np.array_equal(codes_of(codes), c0)
+    for shape, dt in (((300, 70), torch.float32), ((64, 64), torch.bfloat16), ((1, 5), torch.float16), ((0,), torch.float32)):
+        y = (rng.standard_normal(shape) * 3).astype(np.float32)
+        ty = dev(y).to(dt)
+        y = ty.float().cpu().numpy()
+        codes, scale = F8.fp8_quantize_per_tensor(ty)
+        c0, s0 = O.fp8_quantize_per_tensor(y)
+        assert np.float32(scale.item()) == s0 and np.array_equal(codes_of(codes), c0), (shape, dt)
+    z, zs = F8.fp8_quantize_per_tensor(torch.zeros(8, 8, device='cuda'))
+    assert zs.item() == 0 and not codes_of(z).any()
+
+
+@pytest.mark.parametrize('a_shape, b_shape', [[[256, 128], [256, 128]], [[4096, 4096], [4096, 4096]], [[512, 256], [128, 256]],
+                                              [[1, 256], [48, 256]], [[16, 1024], [200, 1024]], [[100, 48], [36, 48]],
+                                              [[300, 272], [260, 272]]])
+def test_matmul_f8_reference_recipe(a_shape, b_shape):
+    # tests/operators_core/test_matmul.py:250-288: randint(-3, 3) inputs; the exact integer result is the answer
+    announce('matmul_f8', a_shape, b_shape)
+    rng = np.random.default_rng(41)
+    ai = rng.integers(-3, 3, a_shape)
+    bi = rng.integers(-3, 3, b_shape)
+    ta, tb = f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32)))
+    exact = ai.astype(np.int64) @ bi.astype(np.int64).T
+    got32 = F8.matmul_f8(ta, tb, output_dtype='float32')
+    assert np.array_equal(host(got32).astype(np.int64), exact)
+    got8 = F8.matmul_f8(ta, tb)  # default output dtype: the fp8 input type, as in the reference
+    assert got8.dtype == torch.float8_e4m3fn
+    assert np.array_equal(codes_of(got8), O.e4m3_encode(exact.astype(np.float32)))
+    gotb = F8.matmul_f8(ta, tb, output_dtype='bfloat16')
+    assert np.array_equal(host(gotb), O.to_bf16(exact.astype(np.float32)))
+    goth = F8.matmul_f8(ta, tb, output_dtype='f16')
+    with np.errstate(over='ignore'):
+        assert np.array_equal(host(goth), exact.astype(np.float32).astype(np.float16))
+
+
+@pytest.mark.parametrize('a_shape, b_shape', [[[4096, 4096], [4096, 4096]], [[2048, 256], [4096, 256]], [[100, 384], [256, 384]]])
+def test_matmul_f8_scaled_reference_recipe(a_shape, b_shape):
+    # tests/operators_core/test_matmul.py:291-373: integers in [-5, 4], integer scales 1..4, bf16 output; the
+    # expected value is built by pre-multiplying the scales into the operands (exact in int64)
+    announce('matmul_f8_scaled', a_shape, b_shape)
+    rng = np.random.default_rng(42)
+    (m, k), n = a_shape, b_shape[0]
+    ai = rng.integers(-5, 5, a_shape)
+    bi = rng.integers(-5, 5, b_shape)
+    sa = rng.integers(1, 5, (k // 128, m)).astype(np.float32)
+    sb = rng.integers(1, 5, (n // 128, k // 128)).astype(np.float32)
+    got = F8.matmul_f8_scaled(f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32))),
+                              scale_a=dev(sa), scale_b=dev(sb), output_dtype='float32')
+    a2 = ai.astype(np.int64) * np.repeat(sa.T.astype(np.int64), 128, axis=1)
+    b2 = bi.astype(np.int64) * np.repeat(np.repeat(sb.astype(np.int64), 128, axis=0), 128, axis=1)
+    exact = a2 @ b2.T
+    assert np.array_equal(host(got).astype(np.int64), exact)
+    gotb = F8.matmul_f8_scaled(f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32))),
+                               scale_a=dev(sa), scale_b=dev(sb), output_dtype='bfloat16')
+    assert np.array_equal(host(gotb), O.to_bf16(exact.astype(np.float32)))
+    if m <= 128:
+        ref = O.matmul_f8_scaled(O.e4m3_encode(ai.astype(np.float32)), O.e4m3_encode(bi.astype(np.float32)), sa, sb, 'float32')
+        assert np.array_equal(host(got), ref)
+
+
+@pytest.mark.parametrize('m,k,n', [(1, 8192, 8192), (16, 1024, 512), (256, 512, 768), (4096, 8192, 8192), (33, 400, 260)])
+def test_per_tensor_parity(m, k, n):
+    announce('fp8 per-tensor', m, k, n)
+    a32, b32 = O.make_inputs(0, m, k, n)
+    b32 = np.ascontiguousarray(b32.T)  # [N, K]
+    ta, sa = F8.fp8_quantize_per_tensor(dev(a32))
+    tb, sb = F8.fp8_quantize_per_tensor(dev(b32))
+    ac, sa0 = O.fp8_quantize_per_tensor(a32)
+    bc, sb0 = O.fp8_quantize_per_tensor(b32)
+    assert np.array_equal(codes_of(ta), ac) and np.array_equal(codes_of(tb), bc)
+    assert np.float32(sa.item()) == sa0 and np.float32(sb.item()) == sb0
+    got = F8.matmul_f8_per_tensor(ta, tb, sa, sb, 'bfloat16')
+    rows = np.arange(m) if m <= 256 else np.array([0, 15, 16, 255, 256, 1000, 2047, 2048, 4095])
+    ref = O.fp8_matmul_per_tensor(ac[rows], bc, sa0, sb0, 'bfloat16')
+    err = O.max_rel_err(host(got)[rows], ref)
+    print('max_rel_err vs oracle', err)
+    assert err <= TOL and err <= 8e-3  # same codes on both sides: only bf16 output rounding and sum order differ
+    # against the unquantized product the fp8 quantization error itself stays inside the gate
+    want = a32[rows].astype(np.float64) @ b32.astype(np.float64).T
+    print('max_rel_err vs unquantized', O.max_rel_err(host(got)[rows], want))
+
+
+def test_batched_and_strided_operands():
+    announce('fp8 batched')
+    rng = np.random.default_rng(5)
+    ai = rng.integers(-3, 3, (3, 20, 64))
+    bi = rng.integers(-3, 3, (40, 64))
+    ta, tb = f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32)))
+    got = F8.matmul_f8(ta, tb, output_dtype='float32')
+    assert tuple(got.shape) == (3, 20, 40)
+    assert np.array_equal(host(got).astype(np.int64), ai.astype(np.int64) @ bi.astype(np.int64).T)
+    b3 = rng.integers(-3, 3, (3, 40, 64))
+    got = F8.matmul_f8(ta, f8(O.e4m3_encode(b3.astype(np.float32))), output_dtype='float32')
+    assert np.array_equal(host(got).astype(np.int64), np.einsum('bmk,bnk->bmn', ai.astype(np.int64), b3.astype(np.int64)))
+    wide = torch.zeros(20, 256, dtype=torch.uint8, device='cuda')
+    wide[:, 64:128] = ta[0].view(torch.uint8)
+    got = F8.matmul_f8(wide[:, 64:128].view(torch.float8_e4m3fn), tb, output_dtype='float32')  # row stride 256
+    assert np.array_equal(host(got).astype(np.int64), ai[0].astype(np.int64) @ bi.astype(np.int64).T)
+
+
+def test_argument_errors():
+    announce('fp8 errors')
+    a = torch.zeros(4, 64, device='cuda').to(torch.float8_e4m3fn)
+    with pytest.raises(ValueError, match='only supports both operands'):
+        F8.matmul_f8(a, torch.zeros(4, 64, device='cuda'))
+    with pytest.raises(ValueError, match='at least 2 dimensions'):
+        F8.matmul_f8(a[0], a)
+    with pytest.raises(ValueError, match=r'\[\.\.\.,M,K\] and \[\.\.\.,N,K\]'):
+        F8.matmul_f8(a, torch.zeros(4, 32, device='cuda').to(torch.float8_e4m3fn))
+    with pytest.raises(NotImplementedError):
+        F8.matmul_f8(a.to(torch.float8_e5m2), a.to(torch.float8_e5m2))
+    with pytest.raises(ValueError, match='bias is not supported'):
+        F8.matmul_f8_scaled(a, a, torch.ones(1, 4, device='cuda'), torch.ones(1, 1, device='cuda'), bias=torch.ones(4, device='cuda'))
