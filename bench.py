@@ -70,6 +70,8 @@ def main():
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--pmc-calibration', action='store_true',
+                    help='short run for `rocprofv3 --pmc`: a few 64 MiB device copies of known traffic, then one pass over the GEMV ring')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: the quantized-matmul path is built and measured on a single MI355X '
@@ -96,6 +98,20 @@ def main():
 
     def launch(i, st):
         ffi.call('hidet_symmetric_quant_matmul_f16_i8', a, ws[i], ss[i], outs[i], 1, K, N, K, 0, work, work.numel(), st)
+
+    if args.pmc_calibration:
+        src = torch.empty(64 << 20, dtype=torch.uint8, device=device).random_(0, 255)
+        dst = torch.empty_like(src)
+        with torch.cuda.stream(stream):
+            for _ in range(4):
+                dst.copy_(src)  # 64 MiB read + 64 MiB written per dispatch
+            for rep in range(2):
+                for i in range(RING):
+                    launch(i, sptr)
+        stream.synchronize()
+        print(json.dumps({'pmc_calibration': {'copy_bytes': 64 << 20, 'copies': 4, 'gemv_launches': 2 * RING,
+                                              'gemv_algorithmic_bytes': GEMV_BYTES}}))
+        return
 
     # ---- parity of one ring entry against the oracle, before anything is timed --------------------------
     from oracle import clib
