@@ -4,7 +4,7 @@
 namespace qmm {
 void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                          int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream);
-bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t k, int64_t n, int64_t lda);
+bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda);
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, hipStream_t stream);
 }
@@ -25,7 +25,7 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     // Up to 64 rows the weight stream dominates: 16 rows per pass of the bandwidth-bound kernel.  Beyond
     // that the MFMA GEMM (128-row tiles) wins.
-    if (m > 64 && k > 0 && gemm_w8a16_supported(a, w, c, k, n, lda))
+    if (m > 64 && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
         gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, stream);
     else
         skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);
