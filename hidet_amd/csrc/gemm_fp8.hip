@@ -53,7 +53,7 @@ __device__ __forceinline__ void store4(void *c, int64_t idx, float4_t v) {
 }
 
 template <int OUT>
-__global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda,
+__global__ __launch_bounds__(kThreads, 1) void gemm_fp8_staged_kernel(const uint8_t *__restrict__ a, int64_t lda,
                                                                const uint8_t *__restrict__ b, int64_t ldb,
                                                                void *__restrict__ c, int m, int n, int k,
                                                                const float *__restrict__ scale_a,
@@ -155,6 +155,253 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
     }
 }
 
+// ---- fast path: K a multiple of 128, 16-byte aligned rows, tensors below 1 GiB -------------------------------
+// Same 256x256 tile and swizzled LDS layout, but:
+//  * both operand tiles go global -> LDS directly (buffer_load ... lds: no staging registers, no ds_write; the
+//    chunk swizzle is applied on the global side);
+//  * LDS holds a ring of three A tiles and two B tiles (160 KiB). A wave reads all eight B fragments of a k-step
+//    up front, so a B slot is free again after the first of the eight row blocks; A fragments stream through
+//    the step. With two barriers per step - P after row block 0 (B slot free -> issue B of step s+2) and L before
+//    the MFMAs of row block 7 (A slot free -> issue A of step s+3; loads of step s+1 confirmed landed) - every
+//    load is issued about two k-steps (~4000 MFMA cycles) before its first use;
+//  * fragment reads are issued by hand in order of first use, the next step's first fragments during row block
+//    7 of the current one, and each wait is tied to the registers it guards.
+constexpr int kTileChunks = kBM * 8;  // 16-byte chunks of one 256 x 128-byte operand tile
+constexpr int kASlots = 3, kBSlots = 2;
+constexpr int kFastLdsBytes = (kASlots + kBSlots) * kTileChunks * 16;  // 160 KiB
+static_assert(kBM == kBN, "A and B tiles share the slot size");
+
+template <int OFFSET>
+__device__ __forceinline__ int4v_t lds_read_b128_early(uint32_t byte_addr) {
+    int4v_t v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(byte_addr), "n"(OFFSET));
+    return v;
+}
+// Wait until at most NEWER LDS reads issued after the ones producing lo/hi are outstanding.
+template <int NEWER>
+__device__ __forceinline__ void lds_wait_keep_newer(int4v_t &lo, int4v_t &hi) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(NEWER));
+}
+__device__ __forceinline__ void buffer_load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint4 *lds_dst, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
+}
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+
+__device__ __forceinline__ float4_t mfma_fp8_k128v(const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1, float4_t acc) {
+    int8v_t rv, cv;
+    rv[0] = r0[0]; rv[1] = r0[1]; rv[2] = r0[2]; rv[3] = r0[3]; rv[4] = r1[0]; rv[5] = r1[1]; rv[6] = r1[2]; rv[7] = r1[3];
+    cv[0] = c0[0]; cv[1] = c0[1]; cv[2] = c0[2]; cv[3] = c0[3]; cv[4] = c1[0]; cv[5] = c1[1]; cv[6] = c1[2]; cv[7] = c1[3];
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+}
+
+template <int OUT>
+__global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda,
+                                                               const uint8_t *__restrict__ b, int64_t ldb,
+                                                               void *__restrict__ c, int m, int n, int k,
+                                                               const float *__restrict__ scale_a,
+                                                               const float *__restrict__ scale_b, int tiles_m, int tiles_n) {
+    extern __shared__ uint4 lds[];  // [kASlots][kTileChunks] A ring, then [kBSlots][kTileChunks] B ring
+
+    const int xcd = blockIdx.x & 7;
+    const int local = blockIdx.x >> 3;
+    const int cb_begin = (tiles_n * xcd) / 8, cb_end = (tiles_n * (xcd + 1)) / 8;
+    if (local >= (cb_end - cb_begin) * tiles_m) return;
+    const int m0 = (local % tiles_m) * kBM;
+    const int n0 = (cb_begin + local / tiles_m) * kBN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int kg = lane >> 4, ls = lane & 15;
+
+    float4_t acc[8][8];  // [row block of a][column block of b]
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a), 0, int(int64_t(m - 1) * lda + k), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b), 0, int(int64_t(n - 1) * ldb + k), 0x00020000);
+    // Load instruction j of a wave fills chunk slots j * 256 + wave * 64 .. + 63 of a tile: tile row
+    // j * 32 + tid / 8, position tid % 8, which holds chunk (tid % 8) ^ (row % 8). Rows past the end of the
+    // tensor get an offset outside the buffer and read as zero.
+    constexpr int kOutside = 0x7FFFFFF0;
+    const int chunk = (tid & 7) ^ ((tid >> 3) & 7);
+    int voff_a[8], voff_b[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int ra = m0 + j * 32 + (tid >> 3), rb = n0 + j * 32 + (tid >> 3);
+        voff_a[j] = ra < m ? int(int64_t(ra) * lda) + chunk * 16 : kOutside;
+        voff_b[j] = rb < n ? int(int64_t(rb) * ldb) + chunk * 16 : kOutside;
+    }
+    // k offsets at and past K stay inside the buffer or read zero; what they fetch is never used
+    auto load_a = [&](int step, int slot) {
+        uint4 *dst = lds + slot * kTileChunks + wave * 64;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) buffer_load_to_lds_b128(rsrc_a, dst + j * kThreads, voff_a[j], step * kBKB);
+    };
+    auto load_b = [&](int step, int slot) {
+        uint4 *dst = lds + (kASlots + slot) * kTileChunks + wave * 64;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) buffer_load_to_lds_b128(rsrc_b, dst + j * kThreads, voff_b[j], step * kBKB);
+    };
+
+    // LDS byte addresses of this lane's two 16-byte fragment halves in block 0 of its wave, slot 0 of each ring;
+    // block i adds i * 16 rows = i * 2048 bytes
+    uint32_t a_addr[2], b_addr[2];
+    {
+        const int ra = wm * 128 + ls, rb = wn * 128 + ls;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            a_addr[h] = uint32_t((ra * 8 + ((2 * kg + h) ^ (ra & 7))) * 16);
+            b_addr[h] = uint32_t(((kASlots * kBM + rb) * 8 + ((2 * kg + h) ^ (rb & 7))) * 16);
+        }
+    }
+    constexpr uint32_t kSlotBytes = kTileChunks * 16;
+
+    const int steps = k / kBKB;
+    load_a(0, 0);
+    load_b(0, 0);
+    load_a(1, 1);
+    load_b(1, 1);
+    load_a(2, 2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(24));
+    __builtin_amdgcn_s_barrier();
+
+    int4v_t bf[8][2], af[3][2];
+    // row block i of a step keeps its A fragment in af[i % 3]
+    bf[0][0] = lds_read_b128_early<0>(b_addr[0]);
+    bf[0][1] = lds_read_b128_early<0>(b_addr[1]);
+    af[0][0] = lds_read_b128_early<0>(a_addr[0]);
+    af[0][1] = lds_read_b128_early<0>(a_addr[1]);
+    bf[1][0] = lds_read_b128_early<1 * 2048>(b_addr[0]); bf[1][1] = lds_read_b128_early<1 * 2048>(b_addr[1]);
+    bf[2][0] = lds_read_b128_early<2 * 2048>(b_addr[0]); bf[2][1] = lds_read_b128_early<2 * 2048>(b_addr[1]);
+    bf[3][0] = lds_read_b128_early<3 * 2048>(b_addr[0]); bf[3][1] = lds_read_b128_early<3 * 2048>(b_addr[1]);
+    bf[4][0] = lds_read_b128_early<4 * 2048>(b_addr[0]); bf[4][1] = lds_read_b128_early<4 * 2048>(b_addr[1]);
+    bf[5][0] = lds_read_b128_early<5 * 2048>(b_addr[0]); bf[5][1] = lds_read_b128_early<5 * 2048>(b_addr[1]);
+    bf[6][0] = lds_read_b128_early<6 * 2048>(b_addr[0]); bf[6][1] = lds_read_b128_early<6 * 2048>(b_addr[1]);
+    bf[7][0] = lds_read_b128_early<7 * 2048>(b_addr[0]); bf[7][1] = lds_read_b128_early<7 * 2048>(b_addr[1]);
+
+    int a_slot = 0, b_slot = 0;  // ring slots of the current step
+    for (int s = 0; s < steps; ++s) {
+        const uint32_t aa0 = a_addr[0] + uint32_t(a_slot) * kSlotBytes, aa1 = a_addr[1] + uint32_t(a_slot) * kSlotBytes;
+        const int a_next = a_slot == kASlots - 1 ? 0 : a_slot + 1, b_next = b_slot ^ 1;
+
+        // ---- row block 0: the reads outstanding are a0, b0 .. b7 of this step (in either order of a0 and b0)
+        lds_wait_keep_newer<14>(bf[0][0], bf[0][1]);
+        lds_wait_keep_newer<14>(af[0][0], af[0][1]);
+        acc[0][0] = mfma_fp8_k128v(bf[0][0], bf[0][1], af[0][0], af[0][1], acc[0][0]);
+        af[1][0] = lds_read_b128_early<1 * 2048>(aa0);
+        af[1][1] = lds_read_b128_early<1 * 2048>(aa1);
+        lds_wait_keep_newer<14>(bf[1][0], bf[1][1]);
+        acc[0][1] = mfma_fp8_k128v(bf[1][0], bf[1][1], af[0][0], af[0][1], acc[0][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait_keep_newer<12>(bf[2][0], bf[2][1]);
+        acc[0][2] = mfma_fp8_k128v(bf[2][0], bf[2][1], af[0][0], af[0][1], acc[0][2]);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait_keep_newer<10>(bf[3][0], bf[3][1]);
+        acc[0][3] = mfma_fp8_k128v(bf[3][0], bf[3][1], af[0][0], af[0][1], acc[0][3]);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait_keep_newer<8>(bf[4][0], bf[4][1]);
+        acc[0][4] = mfma_fp8_k128v(bf[4][0], bf[4][1], af[0][0], af[0][1], acc[0][4]);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait_keep_newer<6>(bf[5][0], bf[5][1]);
+        acc[0][5] = mfma_fp8_k128v(bf[5][0], bf[5][1], af[0][0], af[0][1], acc[0][5]);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait_keep_newer<4>(bf[6][0], bf[6][1]);
+        acc[0][6] = mfma_fp8_k128v(bf[6][0], bf[6][1], af[0][0], af[0][1], acc[0][6]);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_wait_keep_newer<2>(bf[7][0], bf[7][1]);
+        acc[0][7] = mfma_fp8_k128v(bf[7][0], bf[7][1], af[0][0], af[0][1], acc[0][7]);
+        __builtin_amdgcn_sched_barrier(0);
+        // barrier P: every wave holds all B fragments of this step, so its B slot can take step s + 2
+        __builtin_amdgcn_s_barrier();
+        load_b(s + 2, b_slot);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- row blocks 1 .. 6
+        auto row_block = [&](auto i_tag) {
+            constexpr int I = decltype(i_tag)::value;
+            af[(I + 1) % 3][0] = lds_read_b128_early<(I + 1) * 2048>(aa0);
+            af[(I + 1) % 3][1] = lds_read_b128_early<(I + 1) * 2048>(aa1);
+            lds_wait_keep_newer<2>(af[I % 3][0], af[I % 3][1]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[I][j] = mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        row_block(std::integral_constant<int, 1>());
+        row_block(std::integral_constant<int, 2>());
+        row_block(std::integral_constant<int, 3>());
+        row_block(std::integral_constant<int, 4>());
+        row_block(std::integral_constant<int, 5>());
+        row_block(std::integral_constant<int, 6>());
+
+        // ---- row block 7. Barrier L: every wave has read all of this step's A slot, so it can take step s + 3,
+        // and every wave's loads of step s + 1 have landed (the 16 newer ones, A of s + 2 and B of s + 2, may
+        // still be in flight), so the first fragments of step s + 1 can be fetched behind this block's MFMAs.
+        lds_wait_keep_newer<0>(af[1][0], af[1][1]);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(16));
+        __builtin_amdgcn_s_barrier();
+        load_a(s + 3, a_slot);
+        __builtin_amdgcn_sched_barrier(0);
+        {
+            const uint32_t na0 = a_addr[0] + uint32_t(a_next) * kSlotBytes, na1 = a_addr[1] + uint32_t(a_next) * kSlotBytes;
+            const uint32_t nb0 = b_addr[0] + uint32_t(b_next) * kSlotBytes, nb1 = b_addr[1] + uint32_t(b_next) * kSlotBytes;
+            af[0][0] = lds_read_b128_early<0>(na0);
+            af[0][1] = lds_read_b128_early<0>(na1);
+            acc[7][0] = mfma_fp8_k128v(bf[0][0], bf[0][1], af[1][0], af[1][1], acc[7][0]);
+            bf[0][0] = lds_read_b128_early<0 * 2048>(nb0); bf[0][1] = lds_read_b128_early<0 * 2048>(nb1);
+            acc[7][1] = mfma_fp8_k128v(bf[1][0], bf[1][1], af[1][0], af[1][1], acc[7][1]);
+            bf[1][0] = lds_read_b128_early<1 * 2048>(nb0); bf[1][1] = lds_read_b128_early<1 * 2048>(nb1);
+            acc[7][2] = mfma_fp8_k128v(bf[2][0], bf[2][1], af[1][0], af[1][1], acc[7][2]);
+            bf[2][0] = lds_read_b128_early<2 * 2048>(nb0); bf[2][1] = lds_read_b128_early<2 * 2048>(nb1);
+            acc[7][3] = mfma_fp8_k128v(bf[3][0], bf[3][1], af[1][0], af[1][1], acc[7][3]);
+            bf[3][0] = lds_read_b128_early<3 * 2048>(nb0); bf[3][1] = lds_read_b128_early<3 * 2048>(nb1);
+            acc[7][4] = mfma_fp8_k128v(bf[4][0], bf[4][1], af[1][0], af[1][1], acc[7][4]);
+            bf[4][0] = lds_read_b128_early<4 * 2048>(nb0); bf[4][1] = lds_read_b128_early<4 * 2048>(nb1);
+            acc[7][5] = mfma_fp8_k128v(bf[5][0], bf[5][1], af[1][0], af[1][1], acc[7][5]);
+            bf[5][0] = lds_read_b128_early<5 * 2048>(nb0); bf[5][1] = lds_read_b128_early<5 * 2048>(nb1);
+            acc[7][6] = mfma_fp8_k128v(bf[6][0], bf[6][1], af[1][0], af[1][1], acc[7][6]);
+            bf[6][0] = lds_read_b128_early<6 * 2048>(nb0); bf[6][1] = lds_read_b128_early<6 * 2048>(nb1);
+            acc[7][7] = mfma_fp8_k128v(bf[7][0], bf[7][1], af[1][0], af[1][1], acc[7][7]);
+            bf[7][0] = lds_read_b128_early<7 * 2048>(nb0); bf[7][1] = lds_read_b128_early<7 * 2048>(nb1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        a_slot = a_next;
+        b_slot = b_next;
+    }
+    // drain: the look-ahead fragment reads of the step past the end are never used, but their destination
+    // registers must not be reused before they have landed (the wait names every one of them), and LDS must
+    // not be released with tile loads in flight
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(bf[0][0]), "+v"(bf[0][1]), "+v"(bf[1][0]), "+v"(bf[1][1]), "+v"(bf[2][0]), "+v"(bf[2][1]),
+                   "+v"(bf[3][0]), "+v"(bf[3][1]), "+v"(bf[4][0]), "+v"(bf[4][1]), "+v"(bf[5][0]), "+v"(bf[5][1]),
+                   "+v"(bf[6][0]), "+v"(bf[6][1]), "+v"(bf[7][0]), "+v"(bf[7][1]), "+v"(af[0][0]), "+v"(af[0][1]));
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __builtin_amdgcn_sched_barrier(0);
+
+    // acc[i][j][v] = c[m0 + wm*128 + i*16 + ls][n0 + wn*128 + j*16 + 4*kg + v]
+    float alpha = 1.0f;
+    if (scale_a != nullptr) alpha *= *scale_a;
+    if (scale_b != nullptr) alpha *= *scale_b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = m0 + wm * 128 + i * 16 + ls;
+        if (row < m) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int col = n0 + wn * 128 + j * 16 + 4 * kg;
+                if (col < n) {  // n % 4 == 0
+                    float4_t v = acc[i][j];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] *= alpha;
+                    store4<OUT>(c, int64_t(row) * n + col, v);
+                }
+            }
+        }
+    }
+}
+
 // Fallback for shapes the tiled kernel cannot take: one thread per output element.
 template <int OUT>
 __global__ __launch_bounds__(256) void naive_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ b,
@@ -203,11 +450,24 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
         QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
         static bool attr_set = false;  // one flag per output type (the lambda is instantiated per type)
         if (!attr_set) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_kernel<OUT>),
+            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_staged_kernel<OUT>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
             attr_set = true;
         }
-        launch(gemm_fp8_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kLdsBytes), stream, ap, lda, bp, ldb, c,
+        const bool fast = (k % kBKB == 0) && (m - 1) * lda + k <= (int64_t(1) << 30) &&
+                          (n - 1) * ldb + k <= (int64_t(1) << 30);
+        if (fast) {
+            static bool fast_attr_set = false;
+            if (!fast_attr_set) {
+                QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_kernel<OUT>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, kFastLdsBytes));
+                fast_attr_set = true;
+            }
+            launch(gemm_fp8_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kFastLdsBytes), stream, ap, lda, bp, ldb, c,
+                   int(m), int(n), int(k), sa, sb, tiles_m, tiles_n);
+            return;
+        }
+        launch(gemm_fp8_staged_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kLdsBytes), stream, ap, lda, bp, ldb, c,
                int(m), int(n), int(k), sa, sb, tiles_m, tiles_n);
     });
 }

@@ -1,23 +1,25 @@
 // W8A16 prefill GEMM (M > 64): c[m, n] = (sum_k a[m, k] * w[k, n]) * scale[n] on fp16 MFMA with fp32
 // accumulation.
 //
-// The int8 weights never pass through LDS.  Lane (kg, ns) of a wave (kg = lane / 32, ns = lane % 32)
-// loads rows 8kg .. 8kg+7 of a 16-row k-step at columns 4ns .. 4ns+3 (one dword per row); that 8x4
-// byte block holds, for each of its 4 columns, the 8 consecutive k values a 32x32x16 MFMA wants as
+// The int8 weights never pass through LDS.  Lane (kg, ns) of a wave (kg = lane / 16, ns = lane % 16)
+// loads rows 8kg .. 8kg+7 of a 32-row k-step at columns 4ns .. 4ns+3 (one dword per row); that 8x4
+// byte block holds, for each of its 4 columns, the 8 consecutive k values a 16x16x32 MFMA wants as
 // the B operand of output column slot ns.  Byte t of two rows is gathered with one v_perm_b32, one
 // v_xor_b32 turns the pair into two float16 values (0x6400 | (q ^ 0x80) == 1152 + q) and one packed
 // subtract removes the 1152, so the dequantisation is exact and costs 3 VALU ops per 2 weights.  A
-// wave owns RB*32 rows x 128 columns of the output; every dequantised fragment is reused for RB row
-// blocks, and the dequantisation of k-step q+1 is interleaved with the MFMAs of k-step q.
-// (The 32x32x16 form is used because one wave can issue it back to back at ~95 % of the matrix-core
-// rate; the 16x16x32 form reaches ~55 % from one wave.)
+// wave owns 128 rows x 64 columns of the output (128 accumulator registers, two workgroups per CU, so
+// that the second wave of each SIMD runs its MFMAs while the first one dequantises or waits); every
+// dequantised fragment is reused for 8 row blocks.
 //
-// All global reads are buffer loads (scalar base + per-lane constant offset + scalar k offset): no
-// address arithmetic in the loop, and out-of-range rows read as zero.  Weights are prefetched two
-// pipeline stages (128 k) ahead into the register slots they were just dequantised from; the
-// activation tile is staged through LDS (16-byte chunks, XOR-swizzled so the fragment reads are
-// conflict free, double buffered) with its global loads also two stages ahead.  The per-column scale
-// is applied to the fp32 accumulators in the epilogue.
+// The inner loop is laid out by hand in blocks of 4 MFMAs: each block issues the LDS read of the A
+// fragment three blocks ahead (inline ds_read_b128 + a wait tied to the destination registers), does its
+// share of the next k-step's dequantisation (two column pairs) and weight refills, and runs its MFMAs.
+// All global reads are buffer loads (scalar base + per-lane constant offset + scalar k offset): no address
+// arithmetic in the loop, and out-of-range rows read as zero.  Weight rows are refilled one stage (64 k)
+// ahead into the registers they were just dequantised from.  The activation tile goes global -> LDS
+// directly (buffer_load ... lds, no registers) into a three-slot ring of 16-byte chunks XOR-swizzled by
+// row (the swizzle is applied on the global side), two stages ahead; one barrier per 64 k.  The per-column
+// scale is applied to the fp32 accumulators in the epilogue.
 #include "common.h"
 
 namespace qmm {
@@ -48,195 +50,6 @@ __device__ __forceinline__ void buffer_load_to_lds_b128(__amdgpu_buffer_rsrc_t r
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
 }
 
-template <int RB, int WM, int WN>
-struct GemmW8Cfg {
-    static constexpr int kBM = WM * RB * 32;
-    static constexpr int kBN = WN * 128;
-    static constexpr int kThreads = WM * WN * 64;
-    static constexpr int kAChunks = kBM * 8 / kThreads;  // 16-byte chunks of the A stage per thread
-    static constexpr int kLdsBytes = 2 * kBM * 128;
-};
-
-template <int RB, int WM, int WN, int MIN_BLOCKS>
-__global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel(const _Float16 *__restrict__ a, int64_t lda,
-                                                                               const int8_t *__restrict__ w,
-                                                                               const _Float16 *__restrict__ scale,
-                                                                               _Float16 *__restrict__ c, int m, int k, int n,
-                                                                               int tiles_m, int tiles_n) {
-    using Cfg = GemmW8Cfg<RB, WM, WN>;
-    extern __shared__ uint4 lds[];  // [2][kBM * 8] chunks
-
-    // ---- tile of this workgroup: every XCD owns a contiguous range of tile columns and walks it
-    // row-block first, so the workgroups resident on one XCD share a few weight tile columns in L2.
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
-    const int cb_begin = (tiles_n * xcd) / 8, cb_end = (tiles_n * (xcd + 1)) / 8;
-    if (local >= (cb_end - cb_begin) * tiles_m) return;
-    const int cb = cb_begin + local / tiles_m;
-    const int rbk = local % tiles_m;
-    const int m0 = rbk * Cfg::kBM;
-    const int n0 = cb * Cfg::kBN;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-    const int kg = lane >> 5, ns = lane & 31;
-    const int col = n0 + wn * 128 + ns * 4;  // first of this lane's 4 columns
-    const bool col_ok = col < n;              // n % 4 == 0: the 4 columns are in or out together
-
-    float16_t acc[RB][4];
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[rb][t][v] = 0.f;
-
-    // Buffer resources: reads past the end of a or w return zero instead of faulting.
-    const __amdgpu_buffer_rsrc_t rsrc_w =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(w), 0, int(int64_t(k) * n), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<_Float16 *>(a), 0, int((int64_t(m - 1) * lda + k) * 2), 0x00020000);
-
-    // A staging: thread -> chunk (row = tid / 8 + j * kThreads / 8, chunk = tid % 8); byte offsets of the
-    // thread's chunks at k = 0.  Rows past M are pushed out of the buffer range so that they read as zero.
-    const int a_row = tid >> 3, a_chunk = tid & 7;
-    int a_off[Cfg::kAChunks];
-#pragma unroll
-    for (int j = 0; j < Cfg::kAChunks; ++j) {
-        const int row = m0 + a_row + j * (Cfg::kThreads / 8);
-        a_off[j] = row < m ? int((int64_t(row) * lda + a_chunk * 8) * 2) : 0x7FFFFFF0;
-    }
-    // per-lane byte offsets of the 8 rows of a 16-row k-step relative to the k-step's first row
-    int w_off[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) w_off[j] = col_ok ? (kg * 8 + j) * n + col : 0x7FFFFFF0;
-
-    const int stages = k / kBK;  // the launcher guarantees k % kBK == 0
-
-    uint4 a_regs[2][Cfg::kAChunks];  // A chunks of the next two stages, set = stage parity
-    uint32_t w_raw[2][4][8];         // raw int8 rows of the four k-steps of two stages, set = stage parity
-    union BFrag {
-        uint32_t u[4];
-        half2_t h2[4];
-        half8_t h8;
-    };
-    BFrag bq[2][4];      // dequantised B fragments of the current and the next k-step
-    half8_t af[2][RB];   // A fragments of the current and the next k-step
-
-    auto load_a = [&](int st, uint4 (&dst)[Cfg::kAChunks]) {
-#pragma unroll
-        for (int j = 0; j < Cfg::kAChunks; ++j)
-            dst[j] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, a_off[j], st * (kBK * 2), 0));
-    };
-    auto store_a = [&](int buf, const uint4 (&src)[Cfg::kAChunks]) {
-#pragma unroll
-        for (int j = 0; j < Cfg::kAChunks; ++j) {
-            const int r = a_row + j * (Cfg::kThreads / 8);
-            lds[buf * Cfg::kBM * 8 + r * 8 + (a_chunk ^ (r & 7))] = src[j];
-        }
-    };
-    auto load_w = [&](int st, int q, uint32_t (&dst)[8]) {
-        const int soff = (st * kBK + q * 16) * n;  // wave-uniform; past the end every lane reads zero
-#pragma unroll
-        for (int j = 0; j < 8; ++j) dst[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[j], soff, 0);
-    };
-    auto dequant = [&](const uint32_t (&raw)[8], BFrag (&dst)[4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            constexpr uint32_t kZero = 0x0c;
-            const uint32_t sel = (kZero << 24) | (uint32_t(4 + t) << 16) | (kZero << 8) | uint32_t(t);
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                dst[t].u[p] = __builtin_amdgcn_perm(raw[2 * p + 1], raw[2 * p], sel) ^ 0x64806480u;
-                dst[t].h2[p] = dst[t].h2[p] - half2_t{_Float16(1152.0f), _Float16(1152.0f)};
-            }
-        }
-    };
-    auto read_afrag = [&](int buf, int q, half8_t (&dst)[RB]) {
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const int r = (wm * RB + rb) * 32 + ns;
-            dst[rb] = __builtin_bit_cast(half8_t, lds[buf * Cfg::kBM * 8 + r * 8 + ((q * 2 + kg) ^ (r & 7))]);
-        }
-    };
-
-    // One pipeline stage (PAR = stage parity) = four 16-row k-steps.  During the MFMAs of k-step q the next
-    // k-step's weights are dequantised and their raw slot is refilled with the rows two stages ahead.
-    auto stage = [&](int s, auto par_tag) {
-        constexpr int PAR = decltype(par_tag)::value;
-        load_a(s + 2, a_regs[PAR]);  // set PAR was written to LDS at the end of the previous stage
-        read_afrag(PAR, 0, af[0]);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            if (q < 3) {
-                read_afrag(PAR, q + 1, af[(q + 1) & 1]);
-                dequant(w_raw[PAR][q + 1], bq[(q + 1) & 1]);
-                load_w(s + 2, q + 1, w_raw[PAR][q + 1]);
-            } else {
-                dequant(w_raw[PAR ^ 1][0], bq[0]);
-                load_w(s + 3, 0, w_raw[PAR ^ 1][0]);
-            }
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    acc[rb][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[q & 1][rb], bq[q & 1][t].h8, acc[rb][t], 0, 0, 0);
-            // interleave: one MFMA, then a share of the dequantisation / loads of the next k-step
-#pragma unroll
-            for (int i = 0; i < RB * 4; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                            // 1 MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, (48 + RB * 4 - 1) / (RB * 4), 0); // VALU
-                if (i < 8) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                 // 1 VMEM read
-                if (i < RB) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                // 1 DS read
-            }
-        }
-        store_a(PAR ^ 1, a_regs[PAR ^ 1]);  // stage s + 1 into the other LDS buffer (last read in stage s - 1)
-        __syncthreads();
-    };
-
-    // prologue: stage 0 into LDS buffer 0, stage 1 into register set 1, weights of stages 0 and 1 into their sets
-    load_a(0, a_regs[0]);
-    load_a(1, a_regs[1]);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) load_w(0, q, w_raw[0][q]);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) load_w(1, q, w_raw[1][q]);
-    store_a(0, a_regs[0]);
-    dequant(w_raw[0][0], bq[0]);
-    load_w(2, 0, w_raw[0][0]);
-    __syncthreads();
-
-    int s = 0;
-    for (; s + 1 < stages; s += 2) {
-        stage(s, std::integral_constant<int, 0>());
-        stage(s + 1, std::integral_constant<int, 1>());
-    }
-    if (s < stages) stage(s, std::integral_constant<int, 0>());
-
-    // ---- epilogue: scale the fp32 accumulators per column, round to float16, 8-byte stores -----------
-    // acc[rb][t][v] = c[m0 + (wm*RB + rb)*32 + 8*(v/4) + 4*kg + v%4][col + t]
-    if (!col_ok) return;
-    float sc[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) sc[t] = float(scale[col + t]);
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = m0 + (wm * RB + rb) * 32 + 8 * (v >> 2) + 4 * kg + (v & 3);
-            if (row < m) {
-                half4_t o;
-#pragma unroll
-                for (int t = 0; t < 4; ++t) o[t] = _Float16(acc[rb][t][v] * sc[t]);
-                *reinterpret_cast<half4_t *>(c + int64_t(row) * n + col) = o;
-            }
-        }
-}
-
-// ---- the same pipeline on the 16x16x32 MFMA: waves of RB*16 rows x 64 columns (lane (kg, ns) = (lane / 16,
-// lane % 16) loads rows 8kg .. 8kg+7 of a 32-row k-step).  Half the accumulators per wave, so two workgroups
-// fit on a CU and the second wave of each SIMD covers the first one's dequantisation and waits.
 template <int RB, int WM, int WN>
 struct GemmW8Cfg16 {
     static constexpr int kBM = WM * RB * 16;
@@ -415,6 +228,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         stage(s, slot);
         slot = slot == 2 ? 0 : slot + 1;
     }
+    // the activation loads issued for stages past the end are never read, but LDS must not be released with them in flight
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 
     // acc[rb][t][v] = c[m0 + (wm*RB + rb)*16 + 4*kg + v][col + t]
     if (!col_ok) return;
@@ -455,19 +270,6 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
            static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n);
 }
 
-template <int RB, int WM, int WN, int MIN_BLOCKS>
-void launch_cfg(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
-                hipStream_t stream) {
-    using Cfg = GemmW8Cfg<RB, WM, WN>;
-    const int tiles_m = int(cdiv(m, Cfg::kBM)), tiles_n = int(cdiv(n, Cfg::kBN));
-    // every XCD gets floor/ceil(tiles_n / 8) tile columns: size the grid for the largest share
-    const int64_t grid = int64_t(8) * cdiv(tiles_n, 8) * tiles_m;
-    QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-    launch(gemm_w8a16_kernel<RB, WM, WN, MIN_BLOCKS>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
-           static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale),
-           static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n);
-}
-
 }  // namespace
 
 // The MFMA kernel takes K in whole 64-deep stages, 16-byte aligned activation rows, N a multiple of 4 and
@@ -479,14 +281,7 @@ bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m
 
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, hipStream_t stream) {
-    const char *cfg = getenv("QMM_GEMM_CFG");
-    const int which = cfg ? atoi(cfg) : 0;
-    if (which == 1) launch_cfg<4, 1, 2, 1>(a, w, scale, c, m, k, n, lda, stream);       // waves 128 x 128, tile 128 x 256
-    else if (which == 2) launch_cfg<4, 2, 2, 1>(a, w, scale, c, m, k, n, lda, stream);  // waves 128 x 128, tile 256 x 256
-    else if (which == 3) launch_cfg<2, 2, 2, 2>(a, w, scale, c, m, k, n, lda, stream);  // waves 64 x 128, tile 128 x 256
-    else if (which == 4) launch_cfg16<8, 1, 4, 2>(a, w, scale, c, m, k, n, lda, stream);  // 16x16x32: waves 128 x 64, tile 128 x 256
-    else if (which == 5) launch_cfg16<8, 2, 2, 2>(a, w, scale, c, m, k, n, lda, stream);  // 16x16x32: waves 128 x 64, tile 256 x 128
-    else launch_cfg16<8, 1, 4, 2>(a, w, scale, c, m, k, n, lda, stream);
+    launch_cfg16<8, 1, 4, 2>(a, w, scale, c, m, k, n, lda, stream);  // waves 128 x 64, workgroup tile 128 x 256
 }
 
 }  // namespace qmm
