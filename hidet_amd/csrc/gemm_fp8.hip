@@ -10,6 +10,7 @@
 // with the b tile as its row operand: a lane then holds 4 consecutive output columns of one row and
 // stores them together.
 #include "common.h"
+#include "gemm_tiling.h"
 #include "numeric.h"
 
 namespace qmm {
@@ -57,15 +58,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_staged_kernel(const uint
                                                                const uint8_t *__restrict__ b, int64_t ldb,
                                                                void *__restrict__ c, int m, int n, int k,
                                                                const float *__restrict__ scale_a,
-                                                               const float *__restrict__ scale_b, int tiles_m, int tiles_n) {
+                                                               const float *__restrict__ scale_b, int tiles_m, int tiles_n, int xm, int xn) {
     extern __shared__ uint4 lds[];  // [2][kStageChunks]
 
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
-    const int cb_begin = (tiles_n * xcd) / 8, cb_end = (tiles_n * (xcd + 1)) / 8;
-    if (local >= (cb_end - cb_begin) * tiles_m) return;
-    const int m0 = (local % tiles_m) * kBM;
-    const int n0 = (cb_begin + local / tiles_m) * kBN;
+    int tile_m, tile_n;
+    if (!gemm_tile_of_block(tiles_m, tiles_n, xm, xn, &tile_m, &tile_n)) return;
+    const int m0 = tile_m * kBM, n0 = tile_n * kBN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -187,11 +185,14 @@ __device__ __forceinline__ void buffer_load_to_lds_b128(__amdgpu_buffer_rsrc_t r
 }
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
-__device__ __forceinline__ float4_t mfma_fp8_k128v(const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1, float4_t acc) {
-    int8v_t rv, cv;
-    rv[0] = r0[0]; rv[1] = r0[1]; rv[2] = r0[2]; rv[3] = r0[3]; rv[4] = r1[0]; rv[5] = r1[1]; rv[6] = r1[2]; rv[7] = r1[3];
-    cv[0] = c0[0]; cv[1] = c0[1]; cv[2] = c0[2]; cv[3] = c0[3]; cv[4] = c1[0]; cv[5] = c1[1]; cv[6] = c1[2]; cv[7] = c1[3];
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+// acc += r (8 dwords of 32 fp8 per lane) x c, in place in accumulation registers. Written as asm so that the 256
+// accumulator registers of a wave stay where they are (the register allocator otherwise rotates some of them
+// through temporaries, with the wait states that costs) and the MFMAs keep their program order. The scale operand
+// holds E8M0 ones (0x7F bytes); operand formats default to e4m3.
+__device__ __forceinline__ void mfma_fp8_k128v(const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1, float4_t &acc, int unit_scales) {
+    const int8v_t rv = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+    const int8v_t cv = __builtin_shufflevector(c0, c1, 0, 1, 2, 3, 4, 5, 6, 7);
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]" : "+a"(acc) : "v"(rv), "v"(cv), "v"(unit_scales));
 }
 
 template <int OUT>
@@ -199,15 +200,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
                                                                const uint8_t *__restrict__ b, int64_t ldb,
                                                                void *__restrict__ c, int m, int n, int k,
                                                                const float *__restrict__ scale_a,
-                                                               const float *__restrict__ scale_b, int tiles_m, int tiles_n) {
+                                                               const float *__restrict__ scale_b, int tiles_m, int tiles_n, int xm, int xn) {
     extern __shared__ uint4 lds[];  // [kASlots][kTileChunks] A ring, then [kBSlots][kTileChunks] B ring
 
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
-    const int cb_begin = (tiles_n * xcd) / 8, cb_end = (tiles_n * (xcd + 1)) / 8;
-    if (local >= (cb_end - cb_begin) * tiles_m) return;
-    const int m0 = (local % tiles_m) * kBM;
-    const int n0 = (cb_begin + local / tiles_m) * kBN;
+    int tile_m, tile_n;
+    if (!gemm_tile_of_block(tiles_m, tiles_n, xm, xn, &tile_m, &tile_n)) return;
+    const int m0 = tile_m * kBM, n0 = tile_n * kBN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -282,6 +280,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
     bf[6][0] = lds_read_b128_early<6 * 2048>(b_addr[0]); bf[6][1] = lds_read_b128_early<6 * 2048>(b_addr[1]);
     bf[7][0] = lds_read_b128_early<7 * 2048>(b_addr[0]); bf[7][1] = lds_read_b128_early<7 * 2048>(b_addr[1]);
 
+    int unit_scales;
+    asm volatile("v_mov_b32 %0, 0x7f7f7f7f" : "=v"(unit_scales));
     int a_slot = 0, b_slot = 0;  // ring slots of the current step
     for (int s = 0; s < steps; ++s) {
         const uint32_t aa0 = a_addr[0] + uint32_t(a_slot) * kSlotBytes, aa1 = a_addr[1] + uint32_t(a_slot) * kSlotBytes;
@@ -290,29 +290,29 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
         // ---- row block 0: the reads outstanding are a0, b0 .. b7 of this step (in either order of a0 and b0)
         lds_wait_keep_newer<14>(bf[0][0], bf[0][1]);
         lds_wait_keep_newer<14>(af[0][0], af[0][1]);
-        acc[0][0] = mfma_fp8_k128v(bf[0][0], bf[0][1], af[0][0], af[0][1], acc[0][0]);
+        mfma_fp8_k128v(bf[0][0], bf[0][1], af[0][0], af[0][1], acc[0][0], unit_scales);
         af[1][0] = lds_read_b128_early<1 * 2048>(aa0);
         af[1][1] = lds_read_b128_early<1 * 2048>(aa1);
         lds_wait_keep_newer<14>(bf[1][0], bf[1][1]);
-        acc[0][1] = mfma_fp8_k128v(bf[1][0], bf[1][1], af[0][0], af[0][1], acc[0][1]);
+        mfma_fp8_k128v(bf[1][0], bf[1][1], af[0][0], af[0][1], acc[0][1], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         lds_wait_keep_newer<12>(bf[2][0], bf[2][1]);
-        acc[0][2] = mfma_fp8_k128v(bf[2][0], bf[2][1], af[0][0], af[0][1], acc[0][2]);
+        mfma_fp8_k128v(bf[2][0], bf[2][1], af[0][0], af[0][1], acc[0][2], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         lds_wait_keep_newer<10>(bf[3][0], bf[3][1]);
-        acc[0][3] = mfma_fp8_k128v(bf[3][0], bf[3][1], af[0][0], af[0][1], acc[0][3]);
+        mfma_fp8_k128v(bf[3][0], bf[3][1], af[0][0], af[0][1], acc[0][3], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         lds_wait_keep_newer<8>(bf[4][0], bf[4][1]);
-        acc[0][4] = mfma_fp8_k128v(bf[4][0], bf[4][1], af[0][0], af[0][1], acc[0][4]);
+        mfma_fp8_k128v(bf[4][0], bf[4][1], af[0][0], af[0][1], acc[0][4], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         lds_wait_keep_newer<6>(bf[5][0], bf[5][1]);
-        acc[0][5] = mfma_fp8_k128v(bf[5][0], bf[5][1], af[0][0], af[0][1], acc[0][5]);
+        mfma_fp8_k128v(bf[5][0], bf[5][1], af[0][0], af[0][1], acc[0][5], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         lds_wait_keep_newer<4>(bf[6][0], bf[6][1]);
-        acc[0][6] = mfma_fp8_k128v(bf[6][0], bf[6][1], af[0][0], af[0][1], acc[0][6]);
+        mfma_fp8_k128v(bf[6][0], bf[6][1], af[0][0], af[0][1], acc[0][6], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         lds_wait_keep_newer<2>(bf[7][0], bf[7][1]);
-        acc[0][7] = mfma_fp8_k128v(bf[7][0], bf[7][1], af[0][0], af[0][1], acc[0][7]);
+        mfma_fp8_k128v(bf[7][0], bf[7][1], af[0][0], af[0][1], acc[0][7], unit_scales);
         __builtin_amdgcn_sched_barrier(0);
         // barrier P: every wave holds all B fragments of this step, so its B slot can take step s + 2
         __builtin_amdgcn_s_barrier();
@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
             af[(I + 1) % 3][1] = lds_read_b128_early<(I + 1) * 2048>(aa1);
             lds_wait_keep_newer<2>(af[I % 3][0], af[I % 3][1]);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[I][j] = mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j]);
+            for (int j = 0; j < 8; ++j) mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j], unit_scales);
             __builtin_amdgcn_sched_barrier(0);
         };
         row_block(std::integral_constant<int, 1>());
@@ -349,21 +349,21 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
             const uint32_t nb0 = b_addr[0] + uint32_t(b_next) * kSlotBytes, nb1 = b_addr[1] + uint32_t(b_next) * kSlotBytes;
             af[0][0] = lds_read_b128_early<0>(na0);
             af[0][1] = lds_read_b128_early<0>(na1);
-            acc[7][0] = mfma_fp8_k128v(bf[0][0], bf[0][1], af[1][0], af[1][1], acc[7][0]);
+            mfma_fp8_k128v(bf[0][0], bf[0][1], af[1][0], af[1][1], acc[7][0], unit_scales);
             bf[0][0] = lds_read_b128_early<0 * 2048>(nb0); bf[0][1] = lds_read_b128_early<0 * 2048>(nb1);
-            acc[7][1] = mfma_fp8_k128v(bf[1][0], bf[1][1], af[1][0], af[1][1], acc[7][1]);
+            mfma_fp8_k128v(bf[1][0], bf[1][1], af[1][0], af[1][1], acc[7][1], unit_scales);
             bf[1][0] = lds_read_b128_early<1 * 2048>(nb0); bf[1][1] = lds_read_b128_early<1 * 2048>(nb1);
-            acc[7][2] = mfma_fp8_k128v(bf[2][0], bf[2][1], af[1][0], af[1][1], acc[7][2]);
+            mfma_fp8_k128v(bf[2][0], bf[2][1], af[1][0], af[1][1], acc[7][2], unit_scales);
             bf[2][0] = lds_read_b128_early<2 * 2048>(nb0); bf[2][1] = lds_read_b128_early<2 * 2048>(nb1);
-            acc[7][3] = mfma_fp8_k128v(bf[3][0], bf[3][1], af[1][0], af[1][1], acc[7][3]);
+            mfma_fp8_k128v(bf[3][0], bf[3][1], af[1][0], af[1][1], acc[7][3], unit_scales);
             bf[3][0] = lds_read_b128_early<3 * 2048>(nb0); bf[3][1] = lds_read_b128_early<3 * 2048>(nb1);
-            acc[7][4] = mfma_fp8_k128v(bf[4][0], bf[4][1], af[1][0], af[1][1], acc[7][4]);
+            mfma_fp8_k128v(bf[4][0], bf[4][1], af[1][0], af[1][1], acc[7][4], unit_scales);
             bf[4][0] = lds_read_b128_early<4 * 2048>(nb0); bf[4][1] = lds_read_b128_early<4 * 2048>(nb1);
-            acc[7][5] = mfma_fp8_k128v(bf[5][0], bf[5][1], af[1][0], af[1][1], acc[7][5]);
+            mfma_fp8_k128v(bf[5][0], bf[5][1], af[1][0], af[1][1], acc[7][5], unit_scales);
             bf[5][0] = lds_read_b128_early<5 * 2048>(nb0); bf[5][1] = lds_read_b128_early<5 * 2048>(nb1);
-            acc[7][6] = mfma_fp8_k128v(bf[6][0], bf[6][1], af[1][0], af[1][1], acc[7][6]);
+            mfma_fp8_k128v(bf[6][0], bf[6][1], af[1][0], af[1][1], acc[7][6], unit_scales);
             bf[6][0] = lds_read_b128_early<6 * 2048>(nb0); bf[6][1] = lds_read_b128_early<6 * 2048>(nb1);
-            acc[7][7] = mfma_fp8_k128v(bf[7][0], bf[7][1], af[1][0], af[1][1], acc[7][7]);
+            mfma_fp8_k128v(bf[7][0], bf[7][1], af[1][0], af[1][1], acc[7][7], unit_scales);
             bf[7][0] = lds_read_b128_early<7 * 2048>(nb0); bf[7][1] = lds_read_b128_early<7 * 2048>(nb1);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -378,6 +378,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
                    "+v"(bf[3][0]), "+v"(bf[3][1]), "+v"(bf[4][0]), "+v"(bf[4][1]), "+v"(bf[5][0]), "+v"(bf[5][1]),
                    "+v"(bf[6][0]), "+v"(bf[6][1]), "+v"(bf[7][0]), "+v"(bf[7][1]), "+v"(af[0][0]), "+v"(af[0][1]));
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    // the compiler does not see the MFMAs inside the asm: let the last ones retire before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
     // acc[i][j][v] = c[m0 + wm*128 + i*16 + ls][n0 + wn*128 + j*16 + 4*kg + v]
@@ -446,7 +448,8 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
             return;
         }
         const int tiles_m = int(cdiv(m, kBM)), tiles_n = int(cdiv(n, kBN));
-        const int64_t grid = int64_t(8) * cdiv(tiles_n, 8) * tiles_m;
+        const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
+        const int64_t grid = tiling.grid();
         QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
         static bool attr_set = false;  // one flag per output type (the lambda is instantiated per type)
         if (!attr_set) {
@@ -464,11 +467,11 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
                 fast_attr_set = true;
             }
             launch(gemm_fp8_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kFastLdsBytes), stream, ap, lda, bp, ldb, c,
-                   int(m), int(n), int(k), sa, sb, tiles_m, tiles_n);
+                   int(m), int(n), int(k), sa, sb, tiles_m, tiles_n, tiling.xm, tiling.xn);
             return;
         }
         launch(gemm_fp8_staged_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kLdsBytes), stream, ap, lda, bp, ldb, c,
-               int(m), int(n), int(k), sa, sb, tiles_m, tiles_n);
+               int(m), int(n), int(k), sa, sb, tiles_m, tiles_n, tiling.xm, tiling.xn);
     });
 }
 
