@@ -6,7 +6,7 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
                          int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda);
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                       int64_t lda, hipStream_t stream);
+                       int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 }
 
 using namespace qmm;
@@ -26,7 +26,7 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
     // Up to 64 rows the weight stream dominates: 16 rows per pass of the bandwidth-bound kernel.  Beyond
     // that the MFMA GEMM (128-row tiles) wins.
     if (m > 64 && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
-        gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, stream);
+        gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
         skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);
     QMM_ENTRY_END

@@ -111,6 +111,11 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef int int8v_t __attribute__((ext_vector_type(8)));
 typedef int int4v_t __attribute__((ext_vector_type(4)));
+typedef unsigned int uint4v_t __attribute__((ext_vector_type(4)));
+
+// The first 64 KiB of a caller-provided workspace hold arrival counters of cross-workgroup exchanges (always
+// returned to zero by the kernel that used them); scratch for partial results follows.
+constexpr int64_t kCounterBytes = 64 << 10;
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 

@@ -221,10 +221,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a), 0, int(int64_t(m - 1) * lda + k), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b), 0, int(int64_t(n - 1) * ldb + k), 0x00020000);
     // Load instruction j of a wave fills chunk slots j * 256 + wave * 64 .. + 63 of a tile: tile row
-    // j * 32 + tid / 8, position tid % 8, which holds chunk (tid % 8) ^ (row % 8). Rows past the end of the
+    // j * 32 + tid / 8, position tid % 8, which holds chunk (tid % 8) ^ lds_swizzle_key_step2(row). Rows past the end of the
     // tensor get an offset outside the buffer and read as zero.
     constexpr int kOutside = 0x7FFFFFF0;
-    const int chunk = (tid & 7) ^ ((tid >> 3) & 7);
+    const int chunk = (tid & 7) ^ lds_swizzle_key_step2(tid >> 3);  // j * 32 does not change the key
     int voff_a[8], voff_b[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -251,8 +251,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
         const int ra = wm * 128 + ls, rb = wn * 128 + ls;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            a_addr[h] = uint32_t((ra * 8 + ((2 * kg + h) ^ (ra & 7))) * 16);
-            b_addr[h] = uint32_t(((kASlots * kBM + rb) * 8 + ((2 * kg + h) ^ (rb & 7))) * 16);
+            a_addr[h] = uint32_t((ra * 8 + ((2 * kg + h) ^ lds_swizzle_key_step2(ra))) * 16);
+            b_addr[h] = uint32_t(((kASlots * kBM + rb) * 8 + ((2 * kg + h) ^ lds_swizzle_key_step2(rb))) * 16);
         }
     }
     constexpr uint32_t kSlotBytes = kTileChunks * 16;

@@ -21,6 +21,7 @@
 // row (the swizzle is applied on the global side), two stages ahead; one barrier per 64 k.  The per-column
 // scale is applied to the fp32 accumulators in the epilogue.
 #include "common.h"
+#include "gemm_tiling.h"
 
 namespace qmm {
 namespace {
@@ -56,7 +57,8 @@ struct GemmW8Cfg16 {
     static constexpr int kBN = WN * 64;
     static constexpr int kThreads = WM * WN * 64;
     static constexpr int kAChunks = kBM * 8 / kThreads;
-    static constexpr int kLdsBytes = 3 * kBM * 128;  // three-slot ring filled by direct-to-LDS loads
+    static constexpr int kRingBytes = 3 * kBM * 128;  // three-slot ring filled by direct-to-LDS loads
+    static constexpr int kLdsBytes = kRingBytes + 16;  // + the fix-up's flag; the ring must start at LDS address 0
 };
 
 template <int RB, int WM, int WN, int MIN_BLOCKS>
@@ -64,18 +66,34 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
                                                                                  const int8_t *__restrict__ w,
                                                                                  const _Float16 *__restrict__ scale,
                                                                                  _Float16 *__restrict__ c, int m, int k, int n,
-                                                                                 int tiles_m, int tiles_n) {
+                                                                                 int tiles_m, int tiles_n, int xm, int xn,
+                                                                                 int concurrent, int tail_parts, int tail_stride,
+                                                                                 float *__restrict__ partials,
+                                                                                 uint32_t *__restrict__ counters) {
     using Cfg = GemmW8Cfg16<RB, WM, WN>;
-    extern __shared__ uint4 lds[];
+    extern __shared__ uint4 lds[];  // no static LDS in this kernel: fragment reads address the ring from 0
+    int &s_last = *reinterpret_cast<int *>(lds + Cfg::kRingBytes / 16);
 
-    const int xcd = blockIdx.x & 7;
-    const int local = blockIdx.x >> 3;
-    const int cb_begin = (tiles_n * xcd) / 8, cb_end = (tiles_n * (xcd + 1)) / 8;
-    if (local >= (cb_end - cb_begin) * tiles_m) return;
-    const int cb = cb_begin + local / tiles_m;
-    const int rbk = local % tiles_m;
-    const int m0 = rbk * Cfg::kBM;
-    const int n0 = cb * Cfg::kBN;
+    // Work items of an XCD, in launch order: the tiles of its region that fill whole rounds of `concurrent`
+    // workgroups, then the remaining tiles cut into tail_parts K ranges each, so that the last, partly filled round
+    // is shorter (see the fix-up in the epilogue).
+    int tile_m, tile_n, part = 0, parts = 1, tail_slot = 0;
+    {
+        const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, blockIdx.x & 7);
+        const int region_tiles = reg.rows * reg.cols;
+        const int whole = tail_parts > 1 ? (region_tiles / concurrent) * concurrent : region_tiles;
+        int local = blockIdx.x >> 3;
+        if (local >= whole) {
+            const int j = local - whole;
+            local = whole + j / tail_parts;
+            part = j % tail_parts;
+            parts = tail_parts;
+            tail_slot = (blockIdx.x & 7) * tail_stride + j / tail_parts;
+        }
+        if (!gemm_tile_of_region(reg, local, &tile_m, &tile_n)) return;
+    }
+    const int m0 = tile_m * Cfg::kBM;
+    const int n0 = tile_n * Cfg::kBN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -96,7 +114,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         const_cast<_Float16 *>(a), 0, int((int64_t(m - 1) * lda + k) * 2), 0x00020000);
 
     // A staging by direct-to-LDS loads: instruction j of a wave fills the 64 consecutive 16-byte LDS slots
-    // (j * kThreads + wave * 64 .. + 63); slot id holds chunk ((id % 8) ^ (row % 8)) of tile row id / 8, so
+    // (j * kThreads + wave * 64 .. + 63); slot id holds chunk ((id % 8) ^ lds_swizzle_key_step1(row)) of tile row id / 8, so
     // the swizzle is applied on the global side.  Rows past M point outside the buffer and read as zero.
     int a_off[Cfg::kAChunks];
 #pragma unroll
@@ -104,13 +122,14 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         const int id = j * Cfg::kThreads + tid;
         const int r = id >> 3;
         const int row = m0 + r;
-        a_off[j] = row < m ? int((int64_t(row) * lda + ((id & 7) ^ (r & 7)) * 8) * 2) : 0x7FFFFFF0;
+        a_off[j] = row < m ? int((int64_t(row) * lda + ((id & 7) ^ lds_swizzle_key_step1(r)) * 8) * 2) : 0x7FFFFFF0;
     }
     int w_off[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) w_off[j] = col_ok ? (kg * 8 + j) * n + col : 0x7FFFFFF0;
 
     const int stages = k / kBK;
+    const int s_begin = (stages * part) / parts, s_end = (stages * (part + 1)) / parts;
 
     uint32_t w_raw[2][8];  // raw rows of the two k-steps of a stage; each slot is refilled one stage ahead once dequantised
     union BFrag {
@@ -149,7 +168,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     {
         const int r = wm * RB * 16 + ns;
 #pragma unroll
-        for (int q = 0; q < 2; ++q) af_addr[q] = uint32_t((r * 8 + ((q * 4 + kg) ^ (r & 7))) * 16);
+        for (int q = 0; q < 2; ++q) af_addr[q] = uint32_t((r * 8 + ((q * 4 + kg) ^ lds_swizzle_key_step1(r))) * 16);
     }
     auto stage = [&](int s, int slot) {
         load_a(s + 2, slot >= 1 ? slot - 1 : 2);  // slot (s + 2) % 3: last read in stage s - 1
@@ -215,21 +234,63 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         __syncthreads();
     };
 
-    load_a(0, 0);
-    load_a(1, 1);
-    load_w(0, 0, w_raw[0]);
-    load_w(0, 1, w_raw[1]);
+    load_a(s_begin, 0);
+    load_a(s_begin + 1, 1);
+    load_w(s_begin, 0, w_raw[0]);
+    load_w(s_begin, 1, w_raw[1]);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     dequant(w_raw[0], bq[0]);
-    load_w(1, 0, w_raw[0]);
+    load_w(s_begin + 1, 0, w_raw[0]);
     __syncthreads();
 
-    for (int s = 0, slot = 0; s < stages; ++s) {
+    for (int s = s_begin, slot = 0; s < s_end; ++s) {
         stage(s, slot);
         slot = slot == 2 ? 0 : slot + 1;
     }
     // the activation loads issued for stages past the end are never read, but LDS must not be released with them in flight
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+
+    // Fix-up of a tile computed in K ranges: every part writes its fp32 accumulators to the workspace (16 bytes per
+    // lane, agent scope), waits for the writes to be acknowledged and counts itself in; the part that arrives
+    // last reads all of them back in part order - so the sum does not depend on arrival order - and finishes the
+    // tile. The counter goes back to zero for the next launch.
+    if (parts > 1) {
+        const __amdgpu_buffer_rsrc_t rsrc_p = __builtin_amdgcn_make_buffer_rsrc(
+            partials + int64_t(tail_slot) * parts * (Cfg::kBM * Cfg::kBN), 0, parts * Cfg::kBM * Cfg::kBN * 4, 0x00020000);
+        constexpr int kAgentScope = 1 << 4;  // sc1
+        const int lane_off = tid * 16;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v_t, acc[rb][t]), rsrc_p, lane_off,
+                                                       (part * RB * 4 + rb * 4 + t) * (Cfg::kThreads * 16), kAgentScope);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        __syncthreads();
+        if (tid == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(&counters[tail_slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = (old == uint32_t(parts - 1));
+            if (s_last) __hip_atomic_store(&counters[tail_slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!s_last) return;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[rb][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < parts; ++p) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                uint4v_t v[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    v[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, lane_off, (p * RB * 4 + rb * 4 + t) * (Cfg::kThreads * 16),
+                                                                 kAgentScope);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) acc[rb][t] += __builtin_bit_cast(float4_t, v[t]);
+            }
+        }
+    }
 
     // acc[rb][t][v] = c[m0 + (wm*RB + rb)*16 + 4*kg + v][col + t]
     if (!col_ok) return;
@@ -252,10 +313,20 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
 
 template <int RB, int WM, int WN, int MIN_BLOCKS>
 void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
-                  hipStream_t stream) {
+                  void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     using Cfg = GemmW8Cfg16<RB, WM, WN>;
     const int tiles_m = int(cdiv(m, Cfg::kBM)), tiles_n = int(cdiv(n, Cfg::kBN));
-    const int64_t grid = int64_t(8) * cdiv(tiles_n, 8) * tiles_m;
+    constexpr int kConcurrent = 32 * MIN_BLOCKS;  // workgroups an XCD (32 CUs) runs at a time
+    const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
+    // Tail split: at most 4 K ranges of at least 8 stages each, and only with workspace for the partial tiles
+    // (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
+    GemmTail tail = make_gemm_tail(tiling, kConcurrent, 4);
+    while (tail.parts > 1 &&
+           (k / kBK < 8 * tail.parts ||
+            workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
+        --tail.parts;
+    static_assert(8 * kConcurrent * 4 <= kCounterBytes, "one counter per tail tile");
+    const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
     if (Cfg::kLdsBytes > 65536) {
         static bool attr_set = false;
@@ -267,7 +338,8 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     }
     launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale),
-           static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n);
+           static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent, tail.parts, tail.max_tiles,
+           reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
 }
 
 }  // namespace
@@ -280,8 +352,8 @@ bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m
 }
 
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                       int64_t lda, hipStream_t stream) {
-    launch_cfg16<8, 1, 4, 2>(a, w, scale, c, m, k, n, lda, stream);  // waves 128 x 64, workgroup tile 128 x 256
+                       int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    launch_cfg16<8, 1, 4, 2>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);  // waves 128 x 64, workgroup tile 128 x 256
 }
 
 }  // namespace qmm

@@ -9,7 +9,6 @@
 namespace qmm {
 namespace {
 
-constexpr int64_t kCounterBytes = 64 << 10;  // start of the workspace: split-K counters, kept at zero
 
 __global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v) {
     int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;

@@ -9,7 +9,6 @@ namespace qmm {
 constexpr int kSkinnyTileN = 256;
 constexpr int kSkinnyWaves = 4;
 constexpr int kSkinnyRedStride = 272;  // 16 lanes x 17 floats: conflict-free LDS writes
-constexpr int64_t kCounterBytes = 64 << 10;
 constexpr int kMaxSkinnyTiles = int(kCounterBytes / 4);
 
 inline size_t skinny_lds_bytes(int m) { return size_t(kSkinnyWaves) * m * kSkinnyRedStride * sizeof(float); }

@@ -138,7 +138,7 @@ def test_workspace_too_small_is_reported():
 # ---- prefill GEMM (M > 64 goes to the MFMA kernel) ------------------------------------------------------------
 
 @pytest.mark.parametrize('m,k,n', [(128, 64, 256), (256, 512, 512), (65, 128, 64), (200, 200, 260), (130, 72, 12),
-                                   (512, 1024, 1100)])
+                                   (512, 1024, 1100), (256, 2048, 520), (384, 4096, 1100), (1100, 1536, 2100)])
 def test_gemm_exact_on_small_integers(m, k, n):
     announce('w8a16 gemm exact', m, k, n)
     a, q, s = _int_case(m + n, m, k, n)
@@ -178,3 +178,24 @@ def test_gemm_full_size_prefill_rows_sample(n):
     # batch axes are folded into M: [4, 512, K] gives the same numbers as [2048, K]
     got3 = quant.symmetric_quant_matmul(ta.reshape(4, 512, k), tq, ts)
     assert tuple(got3.shape) == (4, 512, n) and torch.equal(got3.reshape(m, n), got)
+
+
+def test_gemm_k_split_matches_unsplit_and_is_deterministic():
+    # With a workspace and fewer tiles than CUs, every tile is computed in K ranges by several workgroups and summed in
+    # a fixed order; without a workspace every tile is computed whole. Both must agree to fp32 rounding, the split
+    # result must not change from run to run, and the arrival counters must be back at zero.
+    m, k, n = 128, 4096, 11008
+    announce('w8a16 gemm k split', m, k, n)
+    a, q, s = _case(1, m, k, n)
+    ta, tq, ts = dev(a), dev(q), dev(s)
+    stream = hidet_amd.ffi.current_stream(ta.device)
+    whole = torch.empty(m, n, dtype=torch.float16, device='cuda')
+    hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8', ta, tq, ts, whole, m, k, n, k, 0, None, 0, stream)
+    assert O.max_rel_err(host(whole), clib.quant_matmul_f32acc(a, q, s)) <= 2e-3
+    first = quant.symmetric_quant_matmul(ta, tq, ts)
+    assert O.max_rel_err(host(first), host(whole)) <= 1e-3
+    for _ in range(3):
+        assert torch.equal(quant.symmetric_quant_matmul(ta, tq, ts), first)
+    ws = hidet_amd.ffi.workspace(ta.device)
+    torch.cuda.synchronize()
+    assert int(ws[: 64 << 10].view(torch.int32).abs().sum()) == 0
