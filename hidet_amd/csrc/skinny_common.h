@@ -134,12 +134,20 @@ __device__ __forceinline__ void skinny_reduce_store(const float4_t (&res)[16], i
     if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
 }
 
-// K split of a skinny launch: enough workgroups to keep about three per CU in flight, slices that are
-// whole multiples of `granule` rows (granule itself a multiple of 128 = 4 waves x one 32-row step).
-inline void skinny_plan(int64_t k, int64_t n, int hint_parts, int granule, int *rows_per_block, int *splits, int *tiles) {
+// K split of a skinny launch. Each workgroup streams a slice of `rows_per_block` weight rows (a whole multiple of
+// `granule` = 4 waves x one 32-row step) of its 256-column tile. Measured on K = 4096 .. 11008 and N = 4096 .. 12288:
+// slices of about 128 KiB (192 KiB for more than 8 activation rows, whose partial tiles cost more to exchange) are
+// fastest - shorter ones pay for the partial-tile exchange, longer ones leave too few workgroups to keep HBM busy -
+// and narrow outputs get more splits so that at least ~128 workgroups run. `hint_parts` > 0 forces the split count.
+inline void skinny_plan(int64_t m, int64_t k, int64_t n, int tile_row_bytes, int hint_parts, int granule, int *rows_per_block,
+                        int *splits, int *tiles) {
     const int64_t t = cdiv(n, kSkinnyTileN);
-    int64_t want = hint_parts > 0 ? hint_parts : std::max<int64_t>(1, (768 + t / 2) / t);
-    want = std::min<int64_t>(want, cdiv(k, granule));
+    int64_t want = hint_parts;
+    if (want <= 0) {
+        const int64_t slice_rows = (m > 8 ? (192 << 10) : (128 << 10)) / tile_row_bytes;
+        want = std::max<int64_t>((k + slice_rows / 2) / slice_rows, cdiv(128, t));
+    }
+    want = std::max<int64_t>(1, std::min<int64_t>(want, cdiv(k, granule)));
     const int64_t rpb = cdiv(cdiv(k, want), granule) * granule;
     *rows_per_block = int(rpb);
     *splits = int(cdiv(k, rpb));
