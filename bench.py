@@ -12,6 +12,7 @@ The same JSON line carries
   cpu_baseline  the restated CPU route of the reference (oracle/cpu_baseline.c) on the host cores, on a
                 bounded sample of the same workload;
   prefill       the M = 2048 GEMM of the same weight shape as TFLOP/s (second half of the metric);
+  fp8_prefill   the e4m3 GEMM [4096, 8192] x [8192, 8192]^T -> bf16 with per-tensor scales as TFLOP/s;
   parity        max relative error of one ring entry against the oracle.
 """
 import argparse
@@ -28,6 +29,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_FP8_PEAK_TFLOPS = 5000.0
+# HBM bytes one GEMV launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over the --pmc-calibration
+# run of this file, each scaled by what the same counter reads for a 64 MiB device copy (FETCH_SIZE x 1.999 KiB,
+# WRITE_SIZE x 1.000 KiB per count): 45.69e6 fetched + 0.39e6 written (output and split-K partial tiles).
+GEMV_MEASURED_TRAFFIC_BYTES = 46.08e6
 K, N = 4096, 11008
 RING = 16
 GEMV_BYTES = K * N + 2 * N + 2 * K + 2 * N  # weights + scales + activations + output, each once
@@ -72,6 +78,9 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--pmc-calibration', action='store_true',
                     help='short run for `rocprofv3 --pmc`: a few 64 MiB device copies of known traffic, then one pass over the GEMV ring')
+    ap.add_argument('--data-dependence', action='store_true',
+                    help='time the two GEMM kernels on all-zero operands and on the benchmark operands: the instruction '
+                         'stream is identical, the difference is the clock the chip sustains under its power limit')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: the quantized-matmul path is built and measured on a single MI355X '
@@ -204,6 +213,63 @@ def main():
     prefill_flops = 2.0 * MP * K * N
     prefill_tflops = prefill_flops / (pd.mean() * 1e-6) / 1e12
 
+    # ---- FP8 e4m3 GEMM with per-tensor scales: a [4096, 8192] ~ N(0, 1), b [8192, 8192] ~ N(0, 0.02), bf16 output ----
+    from hidet_amd.graph.ops.matmul import matmul_f8 as f8ops
+    MF, KF, NF = 4096, 8192, 8192
+    gf = torch.Generator(device=device)
+    gf.manual_seed(0)
+    a8, sa = f8ops.fp8_quantize_per_tensor(torch.randn((MF, KF), generator=gf, device=device, dtype=torch.float32))
+    b8s = []
+    for i in range(3):
+        bq, sb = f8ops.fp8_quantize_per_tensor(torch.randn((NF, KF), generator=gf, device=device, dtype=torch.float32) * 0.02)
+        b8s.append((bq, sb))
+    c8 = torch.empty((MF, NF), dtype=torch.bfloat16, device=device)
+
+    def launch_fp8(i):
+        ffi.call('hidet_matmul_f8', a8, b8s[i][0], c8, MF, NF, KF, KF, KF, 2, sa, b8s[i][1], sptr)
+
+    with torch.cuda.stream(stream):
+        for i in range(3):
+            launch_fp8(i)
+    stream.synchronize()
+    rows8 = np.array([0, 255, 256, 2049, 4095])
+    ref8 = O.fp8_matmul_per_tensor(a8.view(torch.uint8).cpu().numpy()[rows8], b8s[2][0].view(torch.uint8).cpu().numpy(),
+                                   float(sa.cpu()), float(b8s[2][1].cpu()), 'float32')
+    fp8_parity = O.max_rel_err(c8.float().cpu().numpy()[rows8], ref8)
+    ev0, ev1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
+    fd = []
+    for rep in range(24):
+        lib.hidet_qmm_arm_timing(ev0, ev1)
+        launch_fp8(rep % 3)
+        lib.hidet_qmm_event_synchronize(ev1)
+        fd.append(lib.hidet_qmm_event_elapsed_ms(ev0, ev1) * 1e3)
+    lib.hidet_qmm_event_destroy(ev0)
+    lib.hidet_qmm_event_destroy(ev1)
+    fd = np.array(fd[4:])
+    fp8_tflops = 2.0 * MF * KF * NF / (fd.mean() * 1e-6) / 1e12
+
+    if args.data_dependence:
+        def timed(fn, reps=24):
+            e0, e1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
+            d = []
+            for rep in range(reps):
+                lib.hidet_qmm_arm_timing(e0, e1)
+                fn(rep)
+                lib.hidet_qmm_event_synchronize(e1)
+                d.append(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3)
+            lib.hidet_qmm_event_destroy(e0)
+            lib.hidet_qmm_event_destroy(e1)
+            return float(np.mean(d[4:]))
+        az, wz = torch.zeros_like(ap), torch.zeros_like(ws[0])
+        a8z, b8z = torch.zeros_like(a8.view(torch.uint8)), torch.zeros_like(b8s[0][0].view(torch.uint8))
+        w8_zero = timed(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', az, wz, ss[0], cp, MP, K, N, K, 0, work,
+                                           work.numel(), sptr))
+        f8_zero = timed(lambda r: ffi.call('hidet_matmul_f8', a8z, b8z, c8, MF, NF, KF, KF, KF, 2, sa, b8s[0][1], sptr))
+        print(json.dumps({'data_dependence': {
+            'w8a16_gemm_us': {'benchmark_operands': round(float(pd.mean()), 2), 'zero_operands': round(w8_zero, 2)},
+            'fp8_gemm_us': {'benchmark_operands': round(float(fd.mean()), 2), 'zero_operands': round(f8_zero, 2)}}}))
+        return
+
     result = {
         'metric': 'w8a16_decode_gemv_bandwidth', 'value': round(value, 1), 'unit': 'GB/s', 'n_gpus': 1,
         'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 5), 'higher_is_better': True,
@@ -212,7 +278,8 @@ def main():
                    'launches_per_step': RING, 'distinct_weight_buffers': RING, 'bytes_per_launch': GEMV_BYTES,
                    'graph_replay': True},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': None,
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': GEMV_MEASURED_TRAFFIC_BYTES,
+                     'algorithmic_bytes': GEMV_BYTES,
                      'kernel': 'skinny_w8a16_kernel', 'kernel_us_mean': round(kernel_us, 3),
                      'kernel_us_min': round(float(durs.min()), 3), 'kernel_us_p50': round(float(np.median(durs)), 3),
                      'launches_timed': int(durs.size)},
@@ -224,6 +291,12 @@ def main():
                     'roofline': {'bound': 'mfma', 'achieved': round(prefill_tflops, 1), 'peak': MFMA_F16_PEAK_TFLOPS,
                                  'unit': 'TFLOP/s', 'frac': round(prefill_tflops / MFMA_F16_PEAK_TFLOPS, 4)},
                     'max_rel_err_vs_oracle_rows_sample': prefill_parity},
+        'fp8_prefill': {'workload': 'FP8 e4m3 GEMM, a[4096,8192] x b[8192,8192]^T, per-tensor f32 scales -> bf16[4096,8192]',
+                        'value': round(fp8_tflops, 1), 'unit': 'TFLOP/s', 'kernel': 'gemm_fp8_kernel',
+                        'kernel_us_mean': round(float(fd.mean()), 2), 'kernel_us_min': round(float(fd.min()), 2),
+                        'roofline': {'bound': 'mfma', 'achieved': round(fp8_tflops, 1), 'peak': MFMA_FP8_PEAK_TFLOPS,
+                                     'unit': 'TFLOP/s', 'frac': round(fp8_tflops / MFMA_FP8_PEAK_TFLOPS, 4)},
+                        'max_rel_err_vs_oracle_rows_sample': fp8_parity, 'tolerance': 3e-2},
         'parity': {'max_rel_err_vs_oracle': parity, 'tolerance': 1e-2, 'graph_replay_matches_eager': replay_ok},
     }
     if not args.no_cpu_baseline:
