@@ -8,7 +8,7 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
 bool gemm_w4a16_supported(const void *a, const void *w, const void *scales, const void *c, int64_t k, int64_t n,
                           int64_t lda, int group);
 void gemm_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
-                       int64_t lda, int group, int dtype, hipStream_t stream);
+                       int64_t lda, int group, int dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 }  // namespace qmm
 
 using namespace qmm;
@@ -31,7 +31,7 @@ HIDET_API void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, 
     QMM_CHECK(a && c && (k == 0 || (w && scales)), "null tensor pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (m > 64 && k > 0 && gemm_w4a16_supported(a, w, scales, c, k, n, lda, group_size))
-        gemm_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, stream);
+        gemm_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, workspace, workspace_bytes, stream);
     else
         skinny_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, parallel_k_parts, workspace, workspace_bytes,
                             stream);

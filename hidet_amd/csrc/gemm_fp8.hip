@@ -169,22 +169,6 @@ constexpr int kASlots = 3, kBSlots = 2;
 constexpr int kFastLdsBytes = (kASlots + kBSlots) * kTileChunks * 16;  // 160 KiB
 static_assert(kBM == kBN, "A and B tiles share the slot size");
 
-template <int OFFSET>
-__device__ __forceinline__ int4v_t lds_read_b128_early(uint32_t byte_addr) {
-    int4v_t v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(byte_addr), "n"(OFFSET));
-    return v;
-}
-// Wait until at most NEWER LDS reads issued after the ones producing lo/hi are outstanding.
-template <int NEWER>
-__device__ __forceinline__ void lds_wait_keep_newer(int4v_t &lo, int4v_t &hi) {
-    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(NEWER));
-}
-__device__ __forceinline__ void buffer_load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint4 *lds_dst, int voff, int soff) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
-}
-constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
-
 // acc += r (8 dwords of 32 fp8 per lane) x c, in place in accumulation registers. Written as asm so that the 256
 // accumulator registers of a wave stay where they are (the register allocator otherwise rotates some of them
 // through temporaries, with the wait states that costs) and the MFMAs keep their program order. The scale operand

@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <cstdint>
 
+#include "common.h"
+
 namespace qmm {
 
 struct GemmTiling {
@@ -97,6 +99,108 @@ __device__ __forceinline__ bool gemm_tile_of_block(int tiles_m, int tiles_n, int
     return gemm_tile_of_region(reg, blockIdx.x >> 3, tile_m, tile_n);
 }
 
+// ---- instruction-level helpers of the hand-scheduled GEMM loops --------------------------------------------------
+
+// s_waitcnt immediate that waits until at most `n` vector-memory operations are outstanding and leaves the other
+// counters alone (gfx9 encoding: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14).
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+
+// LDS fragment read issued by hand so that it can be placed several MFMAs ahead of its use; the matching wait is
+// tied to the destination registers, so nothing that consumes them can be scheduled above it.
+template <int OFFSET>
+__device__ __forceinline__ int4v_t lds_read_b128_early(uint32_t byte_addr) {
+    int4v_t v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(byte_addr), "n"(OFFSET));
+    return v;
+}
+// Wait until at most NEWER LDS reads issued after the one(s) that produce the given registers are outstanding.
+template <int NEWER>
+__device__ __forceinline__ void lds_wait_keep_newer(int4v_t &v) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(NEWER));
+}
+template <int NEWER>
+__device__ __forceinline__ void lds_wait_keep_newer(int4v_t &lo, int4v_t &hi) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(NEWER));
+}
+
+// 16 bytes per lane from a buffer straight into LDS: lane i of the wave writes lds_dst + 16 * i (lds_dst must be
+// wave-uniform), reading buffer offset voff (per lane) + soff (scalar).
+__device__ __forceinline__ void buffer_load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint4 *lds_dst, int voff, int soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
+}
+
+// Work item of this workgroup. The items of an XCD, in launch order: the tiles of its region that fill whole rounds
+// of `concurrent` workgroups, then the remaining tiles cut into tail_parts K ranges each (tail_parts = 1: every tile
+// is one item). `part` of `parts` is the K range, `slot` numbers the split tiles across the chip (fix-up storage).
+struct GemmWorkItem {
+    int tile_m, tile_n, part, parts, slot;
+};
+
+__device__ __forceinline__ bool gemm_work_item(int tiles_m, int tiles_n, int xm, int xn, int concurrent, int tail_parts,
+                                               int tail_stride, GemmWorkItem *item) {
+    const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, blockIdx.x & 7);
+    const int region_tiles = reg.rows * reg.cols;
+    const int whole = tail_parts > 1 ? (region_tiles / concurrent) * concurrent : region_tiles;
+    int local = blockIdx.x >> 3;
+    item->part = 0;
+    item->parts = 1;
+    item->slot = 0;
+    if (local >= whole) {
+        const int j = local - whole;
+        local = whole + j / tail_parts;
+        item->part = j % tail_parts;
+        item->parts = tail_parts;
+        item->slot = (blockIdx.x & 7) * tail_stride + j / tail_parts;
+    }
+    return gemm_tile_of_region(reg, local, &item->tile_m, &item->tile_n);
+}
+
+// Fix-up of a tile computed in K ranges by item.parts workgroups of THREADS threads, each holding R x T float4
+// accumulators per thread. Every part writes its accumulators to the workspace (16 bytes per lane, agent scope),
+// waits for the writes to be acknowledged and counts itself in; the part that arrives last reads all of them back
+// in part order - so the sum does not depend on arrival order - and returns true with the sums in `acc`: it finishes
+// the tile. The others return false. The counter goes back to zero for the next launch. `flag` is one int of LDS.
+template <int THREADS, int R, int T>
+__device__ __forceinline__ bool gemm_k_split_fixup(float4_t (&acc)[R][T], const GemmWorkItem &item,
+                                                   float *__restrict__ partials, uint32_t *__restrict__ counters, int *flag) {
+    constexpr int kTileFloats = THREADS * R * T * 4;
+    constexpr int kAgentScope = 1 << 4;  // sc1
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        partials + int64_t(item.slot) * item.parts * kTileFloats, 0, item.parts * kTileFloats * 4, 0x00020000);
+    const int lane_off = threadIdx.x * 16;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v_t, acc[r][t]), rsrc, lane_off,
+                                                   ((item.part * R + r) * T + t) * (THREADS * 16), kAgentScope);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // vmcnt(0): every store of this lane has been acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(&counters[item.slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = (old == uint32_t(item.parts - 1));
+        if (*flag) __hip_atomic_store(&counters[item.slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!*flag) return false;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < item.parts; ++p) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            uint4v_t v[T];
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                v[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, ((p * R + r) * T + t) * (THREADS * 16), kAgentScope);
+#pragma unroll
+            for (int t = 0; t < T; ++t) acc[r][t] += __builtin_bit_cast(float4_t, v[t]);
+        }
+    }
+    return true;
+}
+
 // Tiles XCD `xcd` owns (host-side twin of gemm_region_of_xcd).
 inline int gemm_region_tiles(const GemmTiling &t, int xcd) {
     const int xr = xcd / t.xn, xc = xcd % t.xn;
@@ -112,18 +216,20 @@ struct GemmTail {
     int64_t grid;   // workgroups to launch
 };
 
-// K ranges are worth their fix-up traffic only while an XCD has fewer tiles than CUs (32): then as many parts (up to
-// max_parts) as keep the busiest XCD at one workgroup per CU. With whole rounds of workgroups in flight the kernels
-// run at the chip's power limit and a shorter last round buys nothing (measured), so the tail stays whole.
-inline GemmTail make_gemm_tail(const GemmTiling &t, int concurrent, int max_parts) {
+// K ranges are worth their fix-up traffic only while an XCD has fewer tiles than `fill` workgroup slots: then as
+// many parts (up to max_parts) as keep the busiest XCD within `fill`. For the int8 GEMM fill = 32, one workgroup per CU:
+// a second co-resident workgroup buys nothing there (measured). The int4 GEMM spends more issue slots on
+// dequantisation than on MFMAs, so a second workgroup per CU overlaps the two and fill = 64 pays. With whole rounds of
+// workgroups in flight the kernels run at the chip's power limit and a shorter last round buys nothing (measured),
+// so then the tail stays whole.
+inline GemmTail make_gemm_tail(const GemmTiling &t, int concurrent, int fill, int max_parts) {
     GemmTail tail{1, 0, t.grid()};
-    constexpr int kCusPerXcd = 32;
     if (t.region_tiles >= concurrent || t.region_tiles == 0) return tail;
     for (int x = 0; x < 8; ++x) {
         const int n = gemm_region_tiles(t, x);
         if (n > tail.max_tiles) tail.max_tiles = n;
     }
-    int parts = kCusPerXcd / t.region_tiles;
+    int parts = fill / t.region_tiles;
     if (parts > max_parts) parts = max_parts;
     tail.parts = parts < 1 ? 1 : parts;
     return tail;

@@ -7,8 +7,16 @@
 // v_cvt_f32_ubyte, one fma gives q * scale = u * scale - 8 * scale in fp32 and v_cvt_pk rounds two
 // of them to the 16-bit type, which is bit for bit the dequantised weight `dtype(q) * scale`.  The eight
 // values of one column over eight rows are the B operand of a 16x16x32 MFMA.  A wave owns RB*16 rows
-// x 128 columns; the activation tile goes through swizzled, double-buffered LDS.
+// x 128 columns.
+//
+// Two kernels.  gemm_w4a16_kernel16 (K a multiple of 64, group size a multiple of 64, tensors addressable with 31-bit
+// offsets) is built like the int8 GEMM: buffer loads without address arithmetic, the activation tile straight into
+// a three-slot LDS ring (buffer_load ... lds) two stages ahead, the A fragments of a k-step read one k-step ahead by
+// hand-placed ds_read_b128, the raw weight rows of a k-step refilled one stage ahead as soon as they are consumed, the
+// group's scales fetched one stage before the group starts, 2D XCD regions and the deterministic K split for grids that
+// leave CUs idle.  gemm_w4a16_kernel (register-staged, double-buffered LDS, every load predicated) takes the rest.
 #include "common.h"
+#include "gemm_tiling.h"
 
 namespace qmm {
 namespace {
@@ -209,6 +217,254 @@ void launch_cfg(const void *a, const void *w, const void *scales, void *c, int64
            static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n);
 }
 
+
+// ---- fast path -------------------------------------------------------------------------------------------------------
+
+template <int RB, int WM, int WN>
+struct GemmW4Cfg16 {
+    static constexpr int kBM = WM * RB * 16;
+    static constexpr int kBN = WN * 128;
+    static constexpr int kThreads = WM * WN * 64;
+    static constexpr int kAChunks = kBM * 8 / kThreads;
+    static constexpr int kRingBytes = 3 * kBM * 128;
+    static constexpr int kLdsBytes = kRingBytes + 16;  // + the fix-up's flag; the ring must start at LDS address 0
+};
+
+template <int DT, int RB, int WM, int WN, int MIN_BLOCKS>
+__global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w4a16_kernel16(
+    const uint16_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ w, const uint16_t *__restrict__ scales,
+    uint16_t *__restrict__ c, int m, int k, int n, int group, int tiles_m, int tiles_n, int xm, int xn, int concurrent,
+    int tail_parts, int tail_stride, float *__restrict__ partials, uint32_t *__restrict__ counters) {
+    using Cfg = GemmW4Cfg16<RB, WM, WN>;
+    using T = W4G<DT>;
+    extern __shared__ uint4 lds[];  // no static LDS in this kernel: fragment reads address the ring from 0
+    int &s_last = *reinterpret_cast<int *>(lds + Cfg::kRingBytes / 16);
+
+    GemmWorkItem item;
+    if (!gemm_work_item(tiles_m, tiles_n, xm, xn, concurrent, tail_parts, tail_stride, &item)) return;
+    const int m0 = item.tile_m * Cfg::kBM;
+    const int n0 = item.tile_n * Cfg::kBN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int kg = lane >> 4, ns = lane & 15;
+    const int col = n0 + wn * 128 + ns * 8;  // first of this lane's 8 columns
+    const bool col_ok = col < n;              // n % 8 == 0
+
+    float4_t acc[RB][8];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[rb][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int row_bytes = n >> 1;
+    const __amdgpu_buffer_rsrc_t rsrc_w =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w), 0, int(int64_t(k) * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(scales), 0, int(int64_t(k / group) * n * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(a), 0, int((int64_t(m - 1) * lda + k) * 2), 0x00020000);
+
+    // activation staging: instruction j of a wave fills the 64 consecutive 16-byte LDS slots
+    // (j * kThreads + wave * 64 .. + 63); slot id holds chunk ((id % 8) ^ key(row)) of tile row id / 8
+    constexpr int kOutside = 0x7FFFFFF0;  // rows / columns past the tensor read as zero
+    int a_off[Cfg::kAChunks];
+#pragma unroll
+    for (int j = 0; j < Cfg::kAChunks; ++j) {
+        const int id = j * Cfg::kThreads + tid;
+        const int r = id >> 3;
+        const int row = m0 + r;
+        a_off[j] = row < m ? int((int64_t(row) * lda + ((id & 7) ^ lds_swizzle_key_step1(r)) * 8) * 2) : kOutside;
+    }
+    int w_off[8];  // row 8kg + j of a k-step, this lane's dword (8 columns)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w_off[j] = col_ok ? (kg * 8 + j) * row_bytes + (col >> 1) : kOutside;
+    const int s_off = col_ok ? col * 2 : kOutside;
+
+    const int stages = k / kBK;
+    const int s_begin = (stages * item.part) / item.parts, s_end = (stages * (item.part + 1)) / item.parts;
+
+    uint32_t w_raw[2][8];    // raw rows of the two k-steps of a stage; refilled one stage ahead once consumed
+    float sc[8], sc8[8];     // scale (/ 16 for odd columns) and -8 * scale of this lane's 8 columns, current group
+    uint4v_t sc_next;        // raw scales of the group that starts with the next stage
+
+    auto load_a = [&](int st, int slot) {
+#pragma unroll
+        for (int j = 0; j < Cfg::kAChunks; ++j)
+            buffer_load_to_lds_b128(rsrc_a, lds + slot * Cfg::kBM * 8 + j * Cfg::kThreads + wave * 64, a_off[j], st * (kBK * 2));
+    };
+    auto load_w = [&](int st, int q) {
+        // the scalar offset is not part of the buffer's range check: never let it point past the tensor (a prefetch
+        // for a stage past the end re-reads the last stage; its values are not used)
+        const int soff = ((st < stages ? st : stages - 1) * kBK + q * 32) * row_bytes;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w_raw[q][j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[j], soff, 0);
+    };
+    auto load_scales = [&](int st) {  // scales of the group stage st lies in (zero past the end)
+        sc_next = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, s_off, ((st * kBK) / group) * n * 2, 0);
+    };
+    auto take_scales = [&]() {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float sv = T::to_f32(uint16_t(sc_next[t >> 1] >> (16 * (t & 1))));
+            sc8[t] = -8.0f * sv;
+            sc[t] = (t & 1) ? sv * 0.0625f : sv;  // odd columns are widened as 16 * u
+        }
+    };
+
+    // LDS byte address of this lane's A fragment for row block 0 of its wave, k-step 0 / 1, ring slot 0
+    uint32_t af_addr[2];
+    {
+        const int r = wm * RB * 16 + ns;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) af_addr[q] = uint32_t((r * 8 + ((q * 4 + kg) ^ lds_swizzle_key_step1(r))) * 16);
+    }
+
+    int4v_t af[2][RB];  // A fragments of the current and of the next k-step
+    auto read_frags = [&](int4v_t (&dst)[RB], uint32_t addr) {
+        static_assert(RB == 4 || RB == 8, "row blocks per wave");
+        dst[0] = lds_read_b128_early<0 * 2048>(addr);
+        dst[1] = lds_read_b128_early<1 * 2048>(addr);
+        dst[2] = lds_read_b128_early<2 * 2048>(addr);
+        dst[3] = lds_read_b128_early<3 * 2048>(addr);
+        if constexpr (RB == 8) {
+            dst[4] = lds_read_b128_early<4 * 2048>(addr);
+            dst[5] = lds_read_b128_early<5 * 2048>(addr);
+            dst[6] = lds_read_b128_early<6 * 2048>(addr);
+            dst[7] = lds_read_b128_early<7 * 2048>(addr);
+        }
+    };
+    auto wait_frags = [&](int4v_t (&f)[RB]) {  // the RB newest reads (the next k-step's) may stay in flight
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) lds_wait_keep_newer<RB>(f[rb]);
+    };
+
+    // One k-step: the A fragments in `cur` are in flight or landed; the reads of the next k-step's fragments go out
+    // first, then for each of the 8 columns of this lane: dequantise its 8 weights, RB MFMAs. Rows 2p, 2p+1 of the raw
+    // block are dead after column 7, so the refill for the next stage is issued then.
+    auto kstep = [&](auto q_tag, int s, uint32_t next_addr) {
+        constexpr int Q = decltype(q_tag)::value;
+        int4v_t(&cur)[RB] = af[Q];
+        int4v_t(&nxt)[RB] = af[Q ^ 1];
+        // nibble ^ 8 = q + 8 = u. ev[j] keeps u of columns 0,2,4,6 of row j in its 4 bytes, od[j] keeps 16 * u of columns
+        // 1,3,5,7 (their nibbles stay in the high half of each byte; sc[] of odd columns holds scale / 16, exact). One
+        // v_cvt_f32_ubyteN then widens a weight without any shift. The empty asm keeps the compiler from re-deriving
+        // each byte from the raw dword with a shift and a mask of its own.
+        uint32_t ev[8], od[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t r = w_raw[Q][j] ^ 0x88888888u;
+            ev[j] = r & 0x0F0F0F0Fu;
+            od[j] = r & 0xF0F0F0F0u;
+            asm volatile("" : "+v"(ev[j]), "+v"(od[j]));
+        }
+        load_w(s + 1, Q);
+        read_frags(nxt, next_addr);  // after the last k-step this reads a slot nobody uses any more; dropped below
+        __builtin_amdgcn_sched_barrier(0);
+        wait_frags(cur);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            uint4 b;
+            uint32_t *bp = reinterpret_cast<uint32_t *>(&b);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const uint32_t lo = ((t & 1) ? od[2 * p] : ev[2 * p]) >> (8 * (t >> 1));
+                const uint32_t hi = ((t & 1) ? od[2 * p + 1] : ev[2 * p + 1]) >> (8 * (t >> 1));
+                const float flo = __builtin_fmaf(float(lo & 0xFFu), sc[t], sc8[t]);
+                const float fhi = __builtin_fmaf(float(hi & 0xFFu), sc[t], sc8[t]);
+                bp[p] = T::pack2(flo, fhi);
+            }
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+                acc[rb][t] = T::mfma(__builtin_bit_cast(uint4, cur[rb]), b, acc[rb][t]);
+        }
+    };
+
+    load_a(s_begin, 0);
+    load_a(s_begin + 1, 1);
+    load_w(s_begin, 0);
+    load_w(s_begin, 1);
+    load_scales(s_begin);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    take_scales();
+    __syncthreads();
+    read_frags(af[0], af_addr[0]);
+
+    // The loop body has no branches: the scales of the next stage's group are fetched and converted every stage
+    // (one 16-byte load and 16 VALU ops per lane and stage) rather than at group boundaries only.
+    for (int s = s_begin, slot = 0; s < s_end; ++s) {
+        load_a(s + 2, slot >= 1 ? slot - 1 : 2);  // slot (s + 2) % 3: last read in stage s - 1
+        load_scales(s + 1 < stages ? s + 1 : s);
+        const uint32_t slot_off = uint32_t(slot * Cfg::kBM * 128);
+        const int next_slot = slot == 2 ? 0 : slot + 1;
+        kstep(std::integral_constant<int, 0>(), s, af_addr[1] + slot_off);
+        // Every wave must hold the second k-step's fragments before the barrier (two barriers later their slot is
+        // overwritten), and the activation loads of stage s + 1 (issued one stage ago) must have landed in LDS
+        // before anyone reads them; what this stage issued so far (A chunks, scales, 8 weight rows) may stay in flight.
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) lds_wait_keep_newer<0>(af[1][rb]);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(Cfg::kAChunks + 1 + 8));
+        __syncthreads();
+        kstep(std::integral_constant<int, 1>(), s, af_addr[0] + uint32_t(next_slot * Cfg::kBM * 128));
+        take_scales();
+        slot = next_slot;
+    }
+    // drain: the fragment reads issued for the k-step past the end are not used, but their registers must not be reused
+    // before they have landed, and LDS must not be released with activation loads in flight
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) lds_wait_keep_newer<0>(af[0][rb]);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (item.parts > 1 && !gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last)) return;
+
+    if (!col_ok) return;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int row = m0 + (wm * RB + rb) * 16 + kg * 4 + v;
+            if (row < m) {
+                uint4 o;
+                uint32_t *op = reinterpret_cast<uint32_t *>(&o);
+#pragma unroll
+                for (int t = 0; t < 8; t += 2)
+                    op[t >> 1] = uint32_t(T::from_f32(acc[rb][t][v])) | (uint32_t(T::from_f32(acc[rb][t + 1][v])) << 16);
+                *reinterpret_cast<uint4 *>(c + int64_t(row) * n + col) = o;
+            }
+        }
+}
+
+template <int DT, int RB, int WM, int WN, int MIN_BLOCKS>
+void launch_cfg16(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                  int group, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    using Cfg = GemmW4Cfg16<RB, WM, WN>;
+    const int tiles_m = int(cdiv(m, Cfg::kBM)), tiles_n = int(cdiv(n, Cfg::kBN));
+    constexpr int kConcurrent = 32 * MIN_BLOCKS;
+    const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
+    GemmTail tail = make_gemm_tail(tiling, kConcurrent, kConcurrent, 4);
+    while (tail.parts > 1 &&
+           (k / kBK < 8 * tail.parts ||
+            workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
+        --tail.parts;
+    const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
+    QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
+    if (Cfg::kLdsBytes > 65536) {
+        static bool attr_set = false;
+        if (!attr_set) {
+            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a16_kernel16<DT, RB, WM, WN, MIN_BLOCKS>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
+            attr_set = true;
+        }
+    }
+    launch(gemm_w4a16_kernel16<DT, RB, WM, WN, MIN_BLOCKS>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes),
+           stream, static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
+           static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,
+           tail.parts, tail.max_tiles, reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes),
+           static_cast<uint32_t *>(workspace));
+}
+
 }  // namespace
 
 bool gemm_w4a16_supported(const void *a, const void *w, const void *scales, const void *c, int64_t k, int64_t n,
@@ -218,7 +474,15 @@ bool gemm_w4a16_supported(const void *a, const void *w, const void *scales, cons
 }
 
 void gemm_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
-                       int64_t lda, int group, int dtype, hipStream_t stream) {
+                       int64_t lda, int group, int dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    const bool fast = (k % kBK == 0) && (group % kBK == 0) && k * (n / 2) < (int64_t(1) << 31) - (1 << 20) &&
+                      (m * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20) && (k / group) * n * 2 < (int64_t(1) << 31);
+    if (fast) {
+        // workgroup tile 128 x 256: 4 waves of 64 x 128, two workgroups per CU
+        if (dtype == HIDET_QMM_F16) launch_cfg16<HIDET_QMM_F16, 4, 2, 2, 2>(a, w, scales, c, m, k, n, lda, group, workspace, workspace_bytes, stream);
+        else launch_cfg16<HIDET_QMM_BF16, 4, 2, 2, 2>(a, w, scales, c, m, k, n, lda, group, workspace, workspace_bytes, stream);
+        return;
+    }
     // 128 x 256 tiles (2 waves of 128 x 128) when they fill the chip, 64 x 256 tiles otherwise
     const bool big = cdiv(m, 128) * cdiv(n, 256) >= 512;
     if (dtype == HIDET_QMM_F16) {

@@ -28,29 +28,6 @@ namespace {
 
 constexpr int kBK = 64;  // k extent of one pipeline stage (four 16-deep MFMA steps)
 
-// s_waitcnt immediate that waits until at most `n` vector-memory operations are outstanding and leaves the
-// other counters alone (gfx9 encoding: vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits 15:14).
-constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
-
-// LDS fragment read issued by hand so that it can be placed several MFMAs ahead of its use; the matching wait is
-// tied to the destination registers, so nothing that consumes them can be scheduled above it.
-template <int OFFSET>
-__device__ __forceinline__ int4v_t lds_read_b128_early(uint32_t byte_addr) {
-    int4v_t v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(byte_addr), "n"(OFFSET));
-    return v;
-}
-template <int NEWER>
-__device__ __forceinline__ void lds_wait_keep_newer(int4v_t &v) {
-    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(NEWER));
-}
-
-// 16 bytes per lane from a buffer straight into LDS: lane i of the wave writes lds_dst + 16 * i (lds_dst must
-// be wave-uniform), reading buffer offset voff (per lane) + soff (scalar).
-__device__ __forceinline__ void buffer_load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint4 *lds_dst, int voff, int soff) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
-}
-
 template <int RB, int WM, int WN>
 struct GemmW8Cfg16 {
     static constexpr int kBM = WM * RB * 16;
@@ -74,24 +51,9 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     extern __shared__ uint4 lds[];  // no static LDS in this kernel: fragment reads address the ring from 0
     int &s_last = *reinterpret_cast<int *>(lds + Cfg::kRingBytes / 16);
 
-    // Work items of an XCD, in launch order: the tiles of its region that fill whole rounds of `concurrent`
-    // workgroups, then the remaining tiles cut into tail_parts K ranges each, so that the last, partly filled round
-    // is shorter (see the fix-up in the epilogue).
-    int tile_m, tile_n, part = 0, parts = 1, tail_slot = 0;
-    {
-        const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, blockIdx.x & 7);
-        const int region_tiles = reg.rows * reg.cols;
-        const int whole = tail_parts > 1 ? (region_tiles / concurrent) * concurrent : region_tiles;
-        int local = blockIdx.x >> 3;
-        if (local >= whole) {
-            const int j = local - whole;
-            local = whole + j / tail_parts;
-            part = j % tail_parts;
-            parts = tail_parts;
-            tail_slot = (blockIdx.x & 7) * tail_stride + j / tail_parts;
-        }
-        if (!gemm_tile_of_region(reg, local, &tile_m, &tile_n)) return;
-    }
+    GemmWorkItem item;
+    if (!gemm_work_item(tiles_m, tiles_n, xm, xn, concurrent, tail_parts, tail_stride, &item)) return;
+    const int tile_m = item.tile_m, tile_n = item.tile_n, part = item.part, parts = item.parts;
     const int m0 = tile_m * Cfg::kBM;
     const int n0 = tile_n * Cfg::kBN;
 
@@ -145,7 +107,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
             buffer_load_to_lds_b128(rsrc_a, lds + slot * Cfg::kBM * 8 + j * Cfg::kThreads + wave * 64, a_off[j], st * (kBK * 2));
     };
     auto load_w = [&](int st, int q, uint32_t (&dst)[8]) {
-        const int soff = (st * kBK + q * 32) * n;
+        const int soff = ((st < stages ? st : stages - 1) * kBK + q * 32) * n;
 #pragma unroll
         for (int j = 0; j < 8; ++j) dst[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[j], soff, 0);
     };
@@ -201,7 +163,10 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
                     dst.h2[P] = dst.h2[P] - half2_t{_Float16(1152.0f), _Float16(1152.0f)};
                 }
                 if constexpr (RBI & 1) {  // rows 2P and 2P+1 are consumed: refill them with the rows one stage ahead
-                    const int soff = ((Q == 0 ? s + 1 : s + 2) * kBK + (Q ^ 1) * 32) * n;
+                    // the scalar offset is not part of the buffer's range check: a prefetch for a stage past the end
+                    // re-reads the last stage instead (its values are not used)
+                    const int st = Q == 0 ? s + 1 : s + 2;
+                    const int soff = ((st < stages ? st : stages - 1) * kBK + (Q ^ 1) * 32) * n;
                     w_raw[Q ^ 1][2 * P] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[2 * P], soff, 0);
                     w_raw[Q ^ 1][2 * P + 1] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[2 * P + 1], soff, 0);
                 }
@@ -250,47 +215,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     // the activation loads issued for stages past the end are never read, but LDS must not be released with them in flight
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 
-    // Fix-up of a tile computed in K ranges: every part writes its fp32 accumulators to the workspace (16 bytes per
-    // lane, agent scope), waits for the writes to be acknowledged and counts itself in; the part that arrives
-    // last reads all of them back in part order - so the sum does not depend on arrival order - and finishes the
-    // tile. The counter goes back to zero for the next launch.
-    if (parts > 1) {
-        const __amdgpu_buffer_rsrc_t rsrc_p = __builtin_amdgcn_make_buffer_rsrc(
-            partials + int64_t(tail_slot) * parts * (Cfg::kBM * Cfg::kBN), 0, parts * Cfg::kBM * Cfg::kBN * 4, 0x00020000);
-        constexpr int kAgentScope = 1 << 4;  // sc1
-        const int lane_off = tid * 16;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v_t, acc[rb][t]), rsrc_p, lane_off,
-                                                       (part * RB * 4 + rb * 4 + t) * (Cfg::kThreads * 16), kAgentScope);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
-        __syncthreads();
-        if (tid == 0) {
-            const uint32_t old = __hip_atomic_fetch_add(&counters[tail_slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_last = (old == uint32_t(parts - 1));
-            if (s_last) __hip_atomic_store(&counters[tail_slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads();
-        if (!s_last) return;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (int t = 0; t < 4; ++t) acc[rb][t] = float4_t{0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < parts; ++p) {
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb) {
-                uint4v_t v[4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    v[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, lane_off, (p * RB * 4 + rb * 4 + t) * (Cfg::kThreads * 16),
-                                                                 kAgentScope);
-#pragma unroll
-                for (int t = 0; t < 4; ++t) acc[rb][t] += __builtin_bit_cast(float4_t, v[t]);
-            }
-        }
-    }
+    // a tile computed in K ranges is finished by the part that arrives last (gemm_k_split_fixup)
+    if (parts > 1 && !gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last)) return;
 
     // acc[rb][t][v] = c[m0 + (wm*RB + rb)*16 + 4*kg + v][col + t]
     if (!col_ok) return;
@@ -320,7 +246,7 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
     // Tail split: at most 4 K ranges of at least 8 stages each, and only with workspace for the partial tiles
     // (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
-    GemmTail tail = make_gemm_tail(tiling, kConcurrent, 4);
+    GemmTail tail = make_gemm_tail(tiling, kConcurrent, 32, 4);
     while (tail.parts > 1 &&
            (k / kBK < 8 * tail.parts ||
             workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
