@@ -135,18 +135,16 @@ __device__ __forceinline__ void skinny_reduce_store(const float4_t (&res)[16], i
 }
 
 // K split of a skinny launch. Each workgroup streams a slice of `rows_per_block` weight rows (a whole multiple of
-// `granule` = 4 waves x one 32-row step) of its 256-column tile. Measured on K = 4096 .. 11008 and N = 4096 .. 12288:
-// slices of about 128 KiB (192 KiB for more than 8 activation rows, whose partial tiles cost more to exchange) are
-// fastest - shorter ones pay for the partial-tile exchange, longer ones leave too few workgroups to keep HBM busy -
-// and narrow outputs get more splits so that at least ~128 workgroups run. `hint_parts` > 0 forces the split count.
-inline void skinny_plan(int64_t m, int64_t k, int64_t n, int tile_row_bytes, int hint_parts, int granule, int *rows_per_block,
-                        int *splits, int *tiles) {
+// `granule` = 4 waves x one 32-row step) of its 256-column tile. Measured on K = 4096 .. 11008, N = 4096 .. 12288,
+// M = 1 .. 16, int8 and int4 weights: slices of about `slice_rows` = 512 rows are fastest (768 for int8 weights with more
+// than 8 activation rows, whose partial tiles cost more to exchange) - shorter ones pay for the partial-tile exchange,
+// longer ones leave too few workgroups to keep HBM busy - and narrow outputs get more splits so that at least ~128
+// workgroups run. `hint_parts` > 0 forces the split count.
+inline void skinny_plan(int64_t k, int64_t n, int slice_rows, int hint_parts, int granule, int *rows_per_block, int *splits,
+                        int *tiles) {
     const int64_t t = cdiv(n, kSkinnyTileN);
     int64_t want = hint_parts;
-    if (want <= 0) {
-        const int64_t slice_rows = (m > 8 ? (192 << 10) : (128 << 10)) / tile_row_bytes;
-        want = std::max<int64_t>((k + slice_rows / 2) / slice_rows, cdiv(128, t));
-    }
+    if (want <= 0) want = std::max<int64_t>((k + slice_rows / 2) / slice_rows, cdiv(128, t));
     want = std::max<int64_t>(1, std::min<int64_t>(want, cdiv(k, granule)));
     const int64_t rpb = cdiv(cdiv(k, want), granule) * granule;
     *rows_per_block = int(rpb);

@@ -137,7 +137,7 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
         return;
     }
     int rpb, splits, tiles;
-    skinny_plan(std::min<int64_t>(m, 16), k, n, kTileN, parallel_k_parts, 128, &rpb, &splits, &tiles);
+    skinny_plan(k, n, m > 8 ? 768 : 512, parallel_k_parts, 128, &rpb, &splits, &tiles);
     QMM_CHECK(tiles <= kMaxSkinnyTiles, "N too large for the split-K counters");
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16);
     const int grid = int(cdiv(tiles, 8) * 8 * splits);
