@@ -30,7 +30,9 @@ HIDET_API void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, 
     if (m == 0 || n == 0) return;
     QMM_CHECK(a && c && (k == 0 || (w && scales)), "null tensor pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (m > 64 && k > 0 && gemm_w4a16_supported(a, w, scales, c, k, n, lda, group_size))
+    // one or two 16-row passes of the bandwidth-bound kernel (19 us each at K=4096, N=11008) beat the MFMA GEMM
+    // (46 us up to M=128); beyond 32 rows the GEMM wins
+    if (m > 32 && k > 0 && gemm_w4a16_supported(a, w, scales, c, k, n, lda, group_size))
         gemm_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, workspace, workspace_bytes, stream);
     else
         skinny_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, parallel_k_parts, workspace, workspace_bytes,

@@ -23,9 +23,10 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
     QMM_CHECK(a && w && scale && c, "null tensor pointer");
     QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    // Up to 64 rows the weight stream dominates: 16 rows per pass of the bandwidth-bound kernel.  Beyond
-    // that the MFMA GEMM (128-row tiles) wins.
-    if (m > 64 && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
+    // Up to 16 rows one pass of the bandwidth-bound kernel is fastest (21 us at K=4096, N=11008). Beyond that every 16
+    // rows cost another pass over the weights (36 us at M=17, 79 us at M=64) while the MFMA GEMM with its K split takes
+    // 28 us for any M up to 128.
+    if (m > 16 && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
         gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
         skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);

@@ -1,4 +1,4 @@
-// Group-wise W4A16 GEMM (M > 64): c[m, n] = sum_g scale[g, n] * sum_{k in g} a[m, k] * q[k, n] on
+// Group-wise W4A16 GEMM (M > 32): c[m, n] = sum_g scale[g, n] * sum_{k in g} a[m, k] * q[k, n] on
 // bf16 / fp16 MFMA with fp32 accumulation.
 //
 // As in the int8 GEMM the packed weights go straight from global memory into registers: lane (kg, ns)

@@ -1,4 +1,4 @@
-// W8A16 prefill GEMM (M > 64): c[m, n] = (sum_k a[m, k] * w[k, n]) * scale[n] on fp16 MFMA with fp32
+// W8A16 prefill GEMM (M > 16): c[m, n] = (sum_k a[m, k] * w[k, n]) * scale[n] on fp16 MFMA with fp32
 // accumulation.
 //
 // The int8 weights never pass through LDS.  Lane (kg, ns) of a wave (kg = lane / 16, ns = lane % 16)

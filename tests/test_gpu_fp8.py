@@ -57,7 +57,7 @@ def test_matmul_f8_reference_recipe(a_shape, b_shape):
     ai = rng.integers(-3, 3, a_shape)
     bi = rng.integers(-3, 3, b_shape)
     ta, tb = f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32)))
-    exact = ai.astype(np.int64) @ bi.astype(np.int64).T
+    exact = (ai.astype(np.float64) @ bi.astype(np.float64).T).astype(np.int64)  # float64 BLAS: exact on these integers
     got32 = F8.matmul_f8(ta, tb, output_dtype='float32')
     assert np.array_equal(host(got32).astype(np.int64), exact)
     got8 = F8.matmul_f8(ta, tb)  # default output dtype: the fp8 input type, as in the reference
@@ -70,7 +70,8 @@ def test_matmul_f8_reference_recipe(a_shape, b_shape):
         assert np.array_equal(host(goth), exact.astype(np.float32).astype(np.float16))
 
 
-@pytest.mark.parametrize('a_shape, b_shape', [[[4096, 4096], [4096, 4096]], [[2048, 256], [4096, 256]], [[100, 384], [256, 384]]])
+@pytest.mark.parametrize('a_shape, b_shape', [[[4096, 4096], [4096, 4096]], [[2048, 256], [4096, 256]], [[100, 384], [256, 384]],
+                                              [[16384, 7168], [1536, 7168]]])
 def test_matmul_f8_scaled_reference_recipe(a_shape, b_shape):
     # tests/operators_core/test_matmul.py:291-373: integers in [-5, 4], integer scales 1..4, bf16 output; the
     # expected value is built by pre-multiplying the scales into the operands (exact in int64)
@@ -85,7 +86,7 @@ def test_matmul_f8_scaled_reference_recipe(a_shape, b_shape):
                               scale_a=dev(sa), scale_b=dev(sb), output_dtype='float32')
     a2 = ai.astype(np.int64) * np.repeat(sa.T.astype(np.int64), 128, axis=1)
     b2 = bi.astype(np.int64) * np.repeat(np.repeat(sb.astype(np.int64), 128, axis=0), 128, axis=1)
-    exact = a2 @ b2.T
+    exact = (a2.astype(np.float64) @ b2.astype(np.float64).T).astype(np.int64)  # float64 BLAS: exact on these integers
     assert np.array_equal(host(got).astype(np.int64), exact)
     gotb = F8.matmul_f8_scaled(f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32))),
                                scale_a=dev(sa), scale_b=dev(sb), output_dtype='bfloat16')

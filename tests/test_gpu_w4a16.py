@@ -57,7 +57,8 @@ def test_skinny_parity(m, k, n, g, dtype):
     assert err <= (8e-3 if dtype == 'bfloat16' else 2e-3)  # bf16 output rounding is 2^-9 relative
 
 
-@pytest.mark.parametrize('m,k,n,g', [(128, 256, 256, 128), (65, 128, 264, 32), (512, 4096, 1024, 128), (300, 512, 520, 64)])
+@pytest.mark.parametrize('m,k,n,g', [(128, 256, 256, 128), (65, 128, 264, 32), (512, 4096, 1024, 128), (300, 512, 520, 64),
+                                     (33, 4096, 512, 128), (40, 512, 264, 64), (24, 512, 256, 128)])
 @pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
 def test_gemm_parity(m, k, n, g, dtype):
     announce('w4a16 gemm', m, k, n, g, dtype)

@@ -135,10 +135,12 @@ def test_workspace_too_small_is_reported():
                            hidet_amd.ffi.current_stream(ta.device))
 
 
-# ---- prefill GEMM (M > 64 goes to the MFMA kernel) ------------------------------------------------------------
+# ---- prefill GEMM (M > 16 goes to the MFMA kernel) ------------------------------------------------------------
 
 @pytest.mark.parametrize('m,k,n', [(128, 64, 256), (256, 512, 512), (65, 128, 64), (200, 200, 260), (130, 72, 12),
-                                   (512, 1024, 1100), (256, 2048, 520), (384, 4096, 1100), (1100, 1536, 2100)])
+                                   (512, 1024, 1100), (256, 2048, 520), (384, 4096, 1100), (1100, 1536, 2100),
+                                   (17, 128, 64), (40, 2048, 520), (64, 64, 256),
+                                   (40, 100, 64), (33, 72, 48)])  # the last two: K not a multiple of 64, 16-row passes
 def test_gemm_exact_on_small_integers(m, k, n):
     announce('w8a16 gemm exact', m, k, n)
     a, q, s = _int_case(m + n, m, k, n)
