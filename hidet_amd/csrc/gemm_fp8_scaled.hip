@@ -2,11 +2,19 @@
 //   c[m, n] += (sum_{k in block} a[m, k] * b[n, k]) * scale_a[kb, m] * scale_b[n / 128, kb]
 // with scale_a float32 [K/128, M] (M contiguous) and scale_b float32 [N/128, K/128].
 //
-// Workgroup tile 128 x 128 (one scale_b entry per k block), four waves of 64 x 64, k-step 128 bytes
-// through swizzled double-buffered LDS as in the per-tensor kernel.  Each k block is multiplied into a
-// scratch accumulator (one 16x16x128 MFMA per 16 x 16 block) and folded into the running sum with its
-// two scales on the vector ALU.
+// Each k block is multiplied into a scratch accumulator (one 16x16x128 MFMA per 16 x 16 block, C = 0) and folded into
+// the running sum with its two scales on the vector ALU: one fma per accumulator element and k block, which the MFMA
+// cannot absorb (its built-in block scales are powers of two).
+//
+// gemm_fp8_scaled_kernel8 (tensors below 1 GiB, 16-byte aligned): workgroup tile 256 x 128 (one scale_b entry per k
+// block), eight waves of 64 x 64 - two per SIMD, so that one wave's folding overlaps the other's MFMAs; in a single
+// wave the two do not overlap - operand tiles straight into a three-slot LDS ring (buffer_load ... lds) two k blocks
+// ahead, one barrier per k block, hand-placed fragment reads, the scratch accumulator double-buffered per row block so
+// that the fold of row block i runs behind the MFMAs of row block i + 1. The running sums live in VGPRs (the VALU cannot
+// read accumulation registers). gemm_fp8_scaled_kernel (128 x 128 tile, register-staged double-buffered LDS) takes
+// the rest.
 #include "common.h"
+#include "gemm_tiling.h"
 #include "numeric.h"
 
 namespace qmm {
@@ -139,10 +147,219 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_scaled_kernel(const uint
     }
 }
 
+
+// ---- fast path ---------------------------------------------------------------------------------------------------------
+
+constexpr int kM8 = 256, kN8 = 128;           // workgroup tile
+constexpr int kThreads8 = 512;
+constexpr int kSlotChunks8 = (kM8 + kN8) * 8;  // 16-byte chunks of one k block: A rows then B rows
+constexpr int kLoads8 = kSlotChunks8 / kThreads8;  // 6 direct-to-LDS loads per thread and k block
+constexpr int kLdsBytes8 = 3 * kSlotChunks8 * 16;  // 144 KiB
+
+template <int OUT>
+__device__ __forceinline__ void store4_scaled(void *c, int64_t o, float4_t v) {
+    if (OUT == HIDET_QMM_F32) {
+        *reinterpret_cast<float4_t *>(static_cast<float *>(c) + o) = v;
+    } else if (OUT == HIDET_QMM_BF16) {
+        uint2 w2;
+        w2.x = uint32_t(f32_to_bf16_bits(v[0])) | (uint32_t(f32_to_bf16_bits(v[1])) << 16);
+        w2.y = uint32_t(f32_to_bf16_bits(v[2])) | (uint32_t(f32_to_bf16_bits(v[3])) << 16);
+        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
+    } else if (OUT == HIDET_QMM_F16) {
+        uint2 w2;
+        w2.x = uint32_t(f32_to_f16_bits(v[0])) | (uint32_t(f32_to_f16_bits(v[1])) << 16);
+        w2.y = uint32_t(f32_to_f16_bits(v[2])) | (uint32_t(f32_to_f16_bits(v[3])) << 16);
+        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
+    } else {
+        *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(c) + o) =
+            uint32_t(f32_to_e4m3(v[0])) | (uint32_t(f32_to_e4m3(v[1])) << 8) | (uint32_t(f32_to_e4m3(v[2])) << 16) |
+            (uint32_t(f32_to_e4m3(v[3])) << 24);
+    }
+}
+
+__device__ __forceinline__ float4_t mfma_fp8_k128_fresh(const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1) {
+    const int8v_t rv = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+    const int8v_t cv = __builtin_shufflevector(c0, c1, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+}
+
+template <int OUT>
+__global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
+                                                                        const float *__restrict__ scale_a,
+                                                                        const float *__restrict__ scale_b, void *__restrict__ c,
+                                                                        int m, int n, int k, int tiles_m, int tiles_n, int xm, int xn) {
+    extern __shared__ uint4 lds[];  // [3][kSlotChunks8]; no static LDS: fragment reads address the ring from 0
+    int tile_m, tile_n;
+    if (!gemm_tile_of_block(tiles_m, tiles_n, xm, xn, &tile_m, &tile_n)) return;
+    const int m0 = tile_m * kM8, n0 = tile_n * kN8;
+    const int kblocks = k / 128;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int kg = lane >> 4, ls = lane & 15;
+
+    float4_t total[4][4];  // [row block][column block] of this wave's 64 x 64
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) total[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a), 0, int(int64_t(m) * k), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b), 0, int(int64_t(n) * k), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_sa =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(scale_a), 0, int(int64_t(kblocks) * m * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_sb = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(scale_b), 0, int(int64_t(n / 128) * kblocks * 4), 0x00020000);
+
+    // Load instruction j of a wave fills chunk slots j * 512 + wave * 64 .. + 63 of a k block: tile row j * 64 + tid / 8
+    // (A rows for j < 4, B rows after), position tid % 8, which holds chunk (tid % 8) ^ key(row). Rows past the end of a
+    // tensor get an offset outside the buffer and read as zero.
+    constexpr int kOutside = 0x7FFFFFF0;
+    const int chunk = (tid & 7) ^ lds_swizzle_key_step2(tid >> 3);
+    int voff[kLoads8];
+#pragma unroll
+    for (int j = 0; j < kLoads8; ++j) {
+        const int r = j * 64 + (tid >> 3);
+        if (j < 4) voff[j] = m0 + r < m ? int(int64_t(m0 + r) * k) + chunk * 16 : kOutside;
+        else voff[j] = n0 + r - kM8 < n ? int(int64_t(n0 + r - kM8) * k) + chunk * 16 : kOutside;
+    }
+    auto load_tiles = [&](int kb, int slot) {  // k blocks at and past the end stay inside the buffer or read zero
+        uint4 *dst = lds + slot * kSlotChunks8 + wave * 64;
+#pragma unroll
+        for (int j = 0; j < kLoads8; ++j) buffer_load_to_lds_b128(j < 4 ? rsrc_a : rsrc_b, dst + j * kThreads8, voff[j], kb * 128);
+    };
+    // scales of a k block: the lane's 4 rows (one per row block) and the tile's column block
+    int sa_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = m0 + wm * 64 + i * 16 + ls;
+        sa_off[i] = row < m ? row * 4 : kOutside;
+    }
+    const int sb_off = tile_n * kblocks * 4;
+    float sa_next[4], sb_next;
+    auto load_scales = [&](int kb) {
+        const int kbc = kb < kblocks ? kb : kblocks - 1;  // scalar offsets are not range-checked: stay inside
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sa_next[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, sa_off[i], kbc * m * 4, 0));
+        sb_next = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sb, sb_off, kbc * 4, 0));
+    };
+
+    // LDS byte addresses of this lane's two 16-byte fragment halves in block 0 of its wave, ring slot 0; block i adds
+    // i * 16 rows = i * 2048 bytes
+    uint32_t a_addr[2], b_addr[2];
+    {
+        const int ra = wm * 64 + ls, rb = kM8 + wn * 64 + ls;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            a_addr[h] = uint32_t((ra * 8 + ((2 * kg + h) ^ lds_swizzle_key_step2(ra))) * 16);
+            b_addr[h] = uint32_t((rb * 8 + ((2 * kg + h) ^ lds_swizzle_key_step2(rb))) * 16);
+        }
+    }
+    constexpr uint32_t kSlotBytes = kSlotChunks8 * 16;
+
+    load_scales(0);
+    load_tiles(0, 0);
+    load_tiles(1, 1);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(kLoads8));  // k block 0 has landed; block 1 may be in flight
+    __builtin_amdgcn_s_barrier();
+
+    for (int s = 0, slot = 0; s < kblocks; ++s) {
+        float f[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = sa_next[i] * sb_next;
+        load_scales(s + 1);                           // issued before the tile loads: waiting for them later does not
+        load_tiles(s + 2, slot >= 1 ? slot - 1 : 2);  // wait for these. Slot (s + 2) % 3 was last read in k block s - 1.
+        const uint32_t so = uint32_t(slot) * kSlotBytes;
+        const uint32_t aa0 = a_addr[0] + so, aa1 = a_addr[1] + so, ba0 = b_addr[0] + so, ba1 = b_addr[1] + so;
+        int4v_t bf[4][2], af[4][2];
+        bf[0][0] = lds_read_b128_early<0>(ba0);        bf[0][1] = lds_read_b128_early<0>(ba1);
+        af[0][0] = lds_read_b128_early<0>(aa0);        af[0][1] = lds_read_b128_early<0>(aa1);
+        bf[1][0] = lds_read_b128_early<2048>(ba0);     bf[1][1] = lds_read_b128_early<2048>(ba1);
+        bf[2][0] = lds_read_b128_early<4096>(ba0);     bf[2][1] = lds_read_b128_early<4096>(ba1);
+        bf[3][0] = lds_read_b128_early<6144>(ba0);     bf[3][1] = lds_read_b128_early<6144>(ba1);
+        af[1][0] = lds_read_b128_early<2048>(aa0);     af[1][1] = lds_read_b128_early<2048>(aa1);
+        af[2][0] = lds_read_b128_early<4096>(aa0);     af[2][1] = lds_read_b128_early<4096>(aa1);
+        af[3][0] = lds_read_b128_early<6144>(aa0);     af[3][1] = lds_read_b128_early<6144>(aa1);
+        __builtin_amdgcn_sched_barrier(0);
+        float4_t part[2][4];  // scratch accumulators of two consecutive row blocks
+        // row block 0: fragments arrive in issue order b0, a0, b1, b2, b3 (then a1 .. a3: 6 reads)
+        lds_wait_keep_newer<12>(bf[0][0], bf[0][1]);
+        lds_wait_keep_newer<12>(af[0][0], af[0][1]);
+        part[0][0] = mfma_fp8_k128_fresh(bf[0][0], bf[0][1], af[0][0], af[0][1]);
+        lds_wait_keep_newer<10>(bf[1][0], bf[1][1]);
+        part[0][1] = mfma_fp8_k128_fresh(bf[1][0], bf[1][1], af[0][0], af[0][1]);
+        lds_wait_keep_newer<8>(bf[2][0], bf[2][1]);
+        part[0][2] = mfma_fp8_k128_fresh(bf[2][0], bf[2][1], af[0][0], af[0][1]);
+        lds_wait_keep_newer<6>(bf[3][0], bf[3][1]);
+        part[0][3] = mfma_fp8_k128_fresh(bf[3][0], bf[3][1], af[0][0], af[0][1]);
+        __builtin_amdgcn_sched_barrier(0);
+        auto row_block = [&](auto i_tag) {  // MFMAs of row block I, then the fold of row block I - 1 behind them
+            constexpr int I = decltype(i_tag)::value;
+            lds_wait_keep_newer<2 * (3 - I)>(af[I][0], af[I][1]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) part[I & 1][j] = mfma_fp8_k128_fresh(bf[j][0], bf[j][1], af[I][0], af[I][1]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) total[I - 1][j][v] = __builtin_fmaf(part[(I - 1) & 1][j][v], f[I - 1], total[I - 1][j][v]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        row_block(std::integral_constant<int, 1>());
+        row_block(std::integral_constant<int, 2>());
+        row_block(std::integral_constant<int, 3>());
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) total[3][j][v] = __builtin_fmaf(part[1][j][v], f[3], total[3][j][v]);
+        // the tiles of k block s + 1 (issued one block ago) must have landed before anyone reads them; the 5 scale loads
+        // and 6 tile loads issued in this block may stay in flight
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(5 + kLoads8));
+        __builtin_amdgcn_s_barrier();
+        slot = slot == 2 ? 0 : slot + 1;
+    }
+    // LDS must not be released with tile loads in flight
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = m0 + wm * 64 + i * 16 + ls;
+        if (row >= m) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = n0 + wn * 64 + j * 16 + 4 * kg;
+            if (col >= n) continue;
+            store4_scaled<OUT>(c, int64_t(row) * n + col, total[i][j]);
+        }
+    }
+}
+
 }  // namespace
 
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
                             int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+    const bool fast = m * k <= (int64_t(1) << 30) && n * k <= (int64_t(1) << 30) && (k / 128) * m * 4 < (int64_t(1) << 31) &&
+                      aligned(a, 16) && aligned(b, 16) && aligned(c, 16);
+    if (fast) {
+        const int tiles_m = int(cdiv(m, kM8)), tiles_n = int(n / kN8);
+        const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
+        const int64_t grid = tiling.grid();
+        QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
+        auto go = [&](auto kern) {
+            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes8));
+            launch(kern, dim3(uint32_t(grid)), dim3(kThreads8), size_t(kLdsBytes8), stream, static_cast<const uint8_t *>(a),
+                   static_cast<const uint8_t *>(b), static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
+                   int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn);
+        };
+        switch (out_dtype) {
+            case HIDET_QMM_F32: go(gemm_fp8_scaled_kernel8<HIDET_QMM_F32>); break;
+            case HIDET_QMM_F16: go(gemm_fp8_scaled_kernel8<HIDET_QMM_F16>); break;
+            case HIDET_QMM_BF16: go(gemm_fp8_scaled_kernel8<HIDET_QMM_BF16>); break;
+            case HIDET_QMM_E4M3: go(gemm_fp8_scaled_kernel8<HIDET_QMM_E4M3>); break;
+            default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+        }
+        return;
+    }
     const int tiles_m = int(cdiv(m, kT)), tiles_n = int(n / 128);
     const int64_t grid = int64_t(tiles_m) * tiles_n;
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
