@@ -419,6 +419,9 @@ void dispatch_out(int out_dtype, F &&f) {
 
 }  // namespace
 
+void gemm_fp8_kernel8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                             int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
+
 void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
                      int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
     const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
@@ -443,6 +446,13 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
         }
         const bool fast = (k % kBKB == 0) && (m - 1) * lda + k <= (int64_t(1) << 30) &&
                           (n - 1) * ldb + k <= (int64_t(1) << 30);
+        // 256 x 256 tiles (4 waves, 160 KiB of LDS) move the fewest bytes per flop and win once they fill the chip twice
+        // over (8192^3: 449 vs 516 us); with fewer tiles the 256 x 128, 8-wave kernel has the better occupancy and tile
+        // granularity (2048 x 4096 x 11008: 102 vs 120 us; 512 x 4096 x 11008: 33 vs 57 us).
+        if (fast && int64_t(tiles_m) * tiles_n < 512) {
+            gemm_fp8_kernel8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
+            return;
+        }
         if (fast) {
             static bool fast_attr_set = false;
             if (!fast_attr_set) {

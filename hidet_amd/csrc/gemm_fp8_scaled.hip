@@ -183,11 +183,14 @@ __device__ __forceinline__ float4_t mfma_fp8_k128_fresh(const int4v_t &r0, const
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
 
-template <int OUT>
-__global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
-                                                                        const float *__restrict__ scale_a,
-                                                                        const float *__restrict__ scale_b, void *__restrict__ c,
-                                                                        int m, int n, int k, int tiles_m, int tiles_n, int xm, int xn) {
+// SCALED: scale_a / scale_b are the block scales described at the top of the file. !SCALED: plain a x b^T with optional
+// per-tensor scales (one float each, may be null), applied to the sums in the epilogue.
+template <int OUT, bool SCALED>
+__global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *__restrict__ a, int64_t lda,
+                                                                 const uint8_t *__restrict__ b, int64_t ldb,
+                                                                 const float *__restrict__ scale_a,
+                                                                 const float *__restrict__ scale_b, void *__restrict__ c,
+                                                                 int m, int n, int k, int tiles_m, int tiles_n, int xm, int xn) {
     extern __shared__ uint4 lds[];  // [3][kSlotChunks8]; no static LDS: fragment reads address the ring from 0
     int tile_m, tile_n;
     if (!gemm_tile_of_block(tiles_m, tiles_n, xm, xn, &tile_m, &tile_n)) return;
@@ -205,12 +208,14 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const ui
 #pragma unroll
         for (int j = 0; j < 4; ++j) total[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a), 0, int(int64_t(m) * k), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b), 0, int(int64_t(n) * k), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_sa =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(scale_a), 0, int(int64_t(kblocks) * m * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a), 0, int(int64_t(m - 1) * lda + k), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b), 0, int(int64_t(n - 1) * ldb + k), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_sa = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(scale_a), 0, SCALED ? int(int64_t(kblocks) * m * 4) : 0, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_sb = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(scale_b), 0, int(int64_t(n / 128) * kblocks * 4), 0x00020000);
+        const_cast<float *>(scale_b), 0, SCALED ? int(int64_t(n / 128) * kblocks * 4) : 0, 0x00020000);
 
     // Load instruction j of a wave fills chunk slots j * 512 + wave * 64 .. + 63 of a k block: tile row j * 64 + tid / 8
     // (A rows for j < 4, B rows after), position tid % 8, which holds chunk (tid % 8) ^ key(row). Rows past the end of a
@@ -221,8 +226,8 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const ui
 #pragma unroll
     for (int j = 0; j < kLoads8; ++j) {
         const int r = j * 64 + (tid >> 3);
-        if (j < 4) voff[j] = m0 + r < m ? int(int64_t(m0 + r) * k) + chunk * 16 : kOutside;
-        else voff[j] = n0 + r - kM8 < n ? int(int64_t(n0 + r - kM8) * k) + chunk * 16 : kOutside;
+        if (j < 4) voff[j] = m0 + r < m ? int(int64_t(m0 + r) * lda) + chunk * 16 : kOutside;
+        else voff[j] = n0 + r - kM8 < n ? int(int64_t(n0 + r - kM8) * ldb) + chunk * 16 : kOutside;
     }
     auto load_tiles = [&](int kb, int slot) {  // k blocks at and past the end stay inside the buffer or read zero
         uint4 *dst = lds + slot * kSlotChunks8 + wave * 64;
@@ -237,8 +242,9 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const ui
         sa_off[i] = row < m ? row * 4 : kOutside;
     }
     const int sb_off = tile_n * kblocks * 4;
-    float sa_next[4], sb_next;
+    float sa_next[4] = {1.f, 1.f, 1.f, 1.f}, sb_next = 1.f;
     auto load_scales = [&](int kb) {
+        if constexpr (!SCALED) return;
         const int kbc = kb < kblocks ? kb : kblocks - 1;  // scalar offsets are not range-checked: stay inside
 #pragma unroll
         for (int i = 0; i < 4; ++i) sa_next[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_sa, sa_off[i], kbc * m * 4, 0));
@@ -261,7 +267,7 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const ui
     load_scales(0);
     load_tiles(0, 0);
     load_tiles(1, 1);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(kLoads8));  // k block 0 has landed; block 1 may be in flight
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(kLoads8));  // k block 0 (and its scales) has landed; block 1 may be in flight
     __builtin_amdgcn_s_barrier();
 
     for (int s = 0, slot = 0; s < kblocks; ++s) {
@@ -286,41 +292,58 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const ui
         // row block 0: fragments arrive in issue order b0, a0, b1, b2, b3 (then a1 .. a3: 6 reads)
         lds_wait_keep_newer<12>(bf[0][0], bf[0][1]);
         lds_wait_keep_newer<12>(af[0][0], af[0][1]);
-        part[0][0] = mfma_fp8_k128_fresh(bf[0][0], bf[0][1], af[0][0], af[0][1]);
+        auto mm = [&](float4_t &dst_scaled, float4_t &dst_plain, const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1) {
+            if constexpr (SCALED) dst_scaled = mfma_fp8_k128_fresh(r0, r1, c0, c1);
+            else {
+                const int8v_t rv = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
+                const int8v_t cv = __builtin_shufflevector(c0, c1, 0, 1, 2, 3, 4, 5, 6, 7);
+                dst_plain = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, dst_plain, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+            }
+        };
+        mm(part[0][0], total[0][0], bf[0][0], bf[0][1], af[0][0], af[0][1]);
         lds_wait_keep_newer<10>(bf[1][0], bf[1][1]);
-        part[0][1] = mfma_fp8_k128_fresh(bf[1][0], bf[1][1], af[0][0], af[0][1]);
+        mm(part[0][1], total[0][1], bf[1][0], bf[1][1], af[0][0], af[0][1]);
         lds_wait_keep_newer<8>(bf[2][0], bf[2][1]);
-        part[0][2] = mfma_fp8_k128_fresh(bf[2][0], bf[2][1], af[0][0], af[0][1]);
+        mm(part[0][2], total[0][2], bf[2][0], bf[2][1], af[0][0], af[0][1]);
         lds_wait_keep_newer<6>(bf[3][0], bf[3][1]);
-        part[0][3] = mfma_fp8_k128_fresh(bf[3][0], bf[3][1], af[0][0], af[0][1]);
+        mm(part[0][3], total[0][3], bf[3][0], bf[3][1], af[0][0], af[0][1]);
         __builtin_amdgcn_sched_barrier(0);
         auto row_block = [&](auto i_tag) {  // MFMAs of row block I, then the fold of row block I - 1 behind them
             constexpr int I = decltype(i_tag)::value;
             lds_wait_keep_newer<2 * (3 - I)>(af[I][0], af[I][1]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) part[I & 1][j] = mfma_fp8_k128_fresh(bf[j][0], bf[j][1], af[I][0], af[I][1]);
+            for (int j = 0; j < 4; ++j) mm(part[I & 1][j], total[I][j], bf[j][0], bf[j][1], af[I][0], af[I][1]);
+            if constexpr (SCALED) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) total[I - 1][j][v] = __builtin_fmaf(part[(I - 1) & 1][j][v], f[I - 1], total[I - 1][j][v]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         };
         row_block(std::integral_constant<int, 1>());
         row_block(std::integral_constant<int, 2>());
         row_block(std::integral_constant<int, 3>());
+        if constexpr (SCALED) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int v = 0; v < 4; ++v) total[3][j][v] = __builtin_fmaf(part[1][j][v], f[3], total[3][j][v]);
+        }
         // the tiles of k block s + 1 (issued one block ago) must have landed before anyone reads them; the 5 scale loads
         // and 6 tile loads issued in this block may stay in flight
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(5 + kLoads8));
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((SCALED ? 5 : 0) + kLoads8));
         __builtin_amdgcn_s_barrier();
         slot = slot == 2 ? 0 : slot + 1;
     }
     // LDS must not be released with tile loads in flight
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 
+    float alpha = 1.0f;
+    if constexpr (!SCALED) {
+        if (scale_a != nullptr) alpha *= *scale_a;
+        if (scale_b != nullptr) alpha *= *scale_b;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = m0 + wm * 64 + i * 16 + ls;
@@ -328,36 +351,56 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_scaled_kernel8(const ui
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int col = n0 + wn * 64 + j * 16 + 4 * kg;
-            if (col >= n) continue;
-            store4_scaled<OUT>(c, int64_t(row) * n + col, total[i][j]);
+            if (col >= n) continue;  // n % 4 == 0
+            float4_t v = total[i][j];
+            if constexpr (!SCALED) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] *= alpha;
+            }
+            store4_scaled<OUT>(c, int64_t(row) * n + col, v);
         }
     }
 }
 
 }  // namespace
 
+// Launch of the 8-wave kernel; SCALED selects block scales (scale_a [K/128, M], scale_b [N/128, K/128]) or optional
+// per-tensor scales.
+template <bool SCALED>
+static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ldb, const void *scale_a, const void *scale_b,
+                           void *c, int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+    const int tiles_m = int(cdiv(m, kM8)), tiles_n = int(cdiv(n, kN8));
+    const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
+    const int64_t grid = tiling.grid();
+    QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
+    auto go = [&](auto kern) {
+        QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes8));
+        launch(kern, dim3(uint32_t(grid)), dim3(kThreads8), size_t(kLdsBytes8), stream, static_cast<const uint8_t *>(a), lda,
+               static_cast<const uint8_t *>(b), ldb, static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
+               int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn);
+    };
+    switch (out_dtype) {
+        case HIDET_QMM_F32: go(gemm_fp8_kernel8<HIDET_QMM_F32, SCALED>); break;
+        case HIDET_QMM_F16: go(gemm_fp8_kernel8<HIDET_QMM_F16, SCALED>); break;
+        case HIDET_QMM_BF16: go(gemm_fp8_kernel8<HIDET_QMM_BF16, SCALED>); break;
+        case HIDET_QMM_E4M3: go(gemm_fp8_kernel8<HIDET_QMM_E4M3, SCALED>); break;
+        default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+    }
+}
+
+// a x b^T with optional per-tensor scales on the 256 x 128, 8-wave kernel. The caller has checked: K a multiple of 128,
+// 16-byte aligned rows and pointers, N a multiple of 4, tensors below 1 GiB.
+void gemm_fp8_kernel8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                             int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
+    launch_kernel8<false>(a, lda, b, ldb, scale_a, scale_b, c, m, n, k, out_dtype, stream);
+}
+
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
                             int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
     const bool fast = m * k <= (int64_t(1) << 30) && n * k <= (int64_t(1) << 30) && (k / 128) * m * 4 < (int64_t(1) << 31) &&
                       aligned(a, 16) && aligned(b, 16) && aligned(c, 16);
     if (fast) {
-        const int tiles_m = int(cdiv(m, kM8)), tiles_n = int(n / kN8);
-        const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
-        const int64_t grid = tiling.grid();
-        QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-        auto go = [&](auto kern) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes8));
-            launch(kern, dim3(uint32_t(grid)), dim3(kThreads8), size_t(kLdsBytes8), stream, static_cast<const uint8_t *>(a),
-                   static_cast<const uint8_t *>(b), static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
-                   int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn);
-        };
-        switch (out_dtype) {
-            case HIDET_QMM_F32: go(gemm_fp8_scaled_kernel8<HIDET_QMM_F32>); break;
-            case HIDET_QMM_F16: go(gemm_fp8_scaled_kernel8<HIDET_QMM_F16>); break;
-            case HIDET_QMM_BF16: go(gemm_fp8_scaled_kernel8<HIDET_QMM_BF16>); break;
-            case HIDET_QMM_E4M3: go(gemm_fp8_scaled_kernel8<HIDET_QMM_E4M3>); break;
-            default: QMM_FAIL("unsupported output dtype code " << out_dtype);
-        }
+        launch_kernel8<true>(a, k, b, k, scale_a, scale_b, c, m, n, k, out_dtype, stream);
         return;
     }
     const int tiles_m = int(cdiv(m, kT)), tiles_n = int(n / 128);
