@@ -154,10 +154,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_staged_kernel(const uint
 }
 
 // ---- fast path: K a multiple of 128, 16-byte aligned rows, tensors below 1 GiB -------------------------------
-// Same 256x256 tile and swizzled LDS layout, but:
+// Same 256x256 tile and swizzled LDS layout, eight waves of 128 x 64 (two per SIMD), and:
 //  * both operand tiles go global -> LDS directly (buffer_load ... lds: no staging registers, no ds_write; the
 //    chunk swizzle is applied on the global side);
-//  * LDS holds a ring of three A tiles and two B tiles (160 KiB). A wave reads all eight B fragments of a k-step
+//  * LDS holds a ring of three A tiles and two B tiles (160 KiB). A wave reads all its B fragments of a k-step
 //    up front, so a B slot is free again after the first of the eight row blocks; A fragments stream through
 //    the step. With two barriers per step - P after row block 0 (B slot free -> issue B of step s+2) and L before
 //    the MFMAs of row block 7 (A slot free -> issue A of step s+3; loads of step s+1 confirmed landed) - every
@@ -179,12 +179,28 @@ __device__ __forceinline__ void mfma_fp8_k128v(const int4v_t &r0, const int4v_t 
     asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]" : "+a"(acc) : "v"(rv), "v"(cv), "v"(unit_scales));
 }
 
-template <int OUT>
-__global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda,
-                                                               const uint8_t *__restrict__ b, int64_t ldb,
-                                                               void *__restrict__ c, int m, int n, int k,
-                                                               const float *__restrict__ scale_a,
-                                                               const float *__restrict__ scale_b, int tiles_m, int tiles_n, int xm, int xn) {
+// Compile-time loop: f(std::integral_constant<int, I>()) for I = BEGIN .. END - 1, in order.
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>());
+        static_for<BEGIN + 1, END>(f);
+    }
+}
+
+// WAVES = 4: waves of 128 x 128 (2 x 2), one per SIMD. WAVES = 8: waves of 128 x 64 (2 x 4), two per SIMD, so that a
+// wave stalled on a barrier, an LDS read or a tile load leaves the MFMA unit to the other.
+template <int OUT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda,
+                                                                 const uint8_t *__restrict__ b, int64_t ldb,
+                                                                 void *__restrict__ c, int m, int n, int k,
+                                                                 const float *__restrict__ scale_a,
+                                                                 const float *__restrict__ scale_b, int tiles_m, int tiles_n, int xm, int xn) {
+    static_assert(WAVES == 4 || WAVES == 8, "2 x 2 or 2 x 4 waves");
+    constexpr int kThr = WAVES * 64;
+    constexpr int WN = WAVES / 2;          // waves along N
+    constexpr int NB = 16 / WN;            // 16-column blocks (B fragments) per wave
+    constexpr int kLoads = 2048 / kThr;    // direct-to-LDS loads per thread and operand tile
     extern __shared__ uint4 lds[];  // [kASlots][kTileChunks] A ring, then [kBSlots][kTileChunks] B ring
 
     int tile_m, tile_n;
@@ -193,26 +209,26 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int kg = lane >> 4, ls = lane & 15;
 
-    float4_t acc[8][8];  // [row block of a][column block of b]
+    float4_t acc[8][NB];  // [row block of a][column block of b]
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < NB; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a), 0, int(int64_t(m - 1) * lda + k), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b), 0, int(int64_t(n - 1) * ldb + k), 0x00020000);
-    // Load instruction j of a wave fills chunk slots j * 256 + wave * 64 .. + 63 of a tile: tile row
-    // j * 32 + tid / 8, position tid % 8, which holds chunk (tid % 8) ^ lds_swizzle_key_step2(row). Rows past the end of the
-    // tensor get an offset outside the buffer and read as zero.
+    // Load instruction j of a wave fills chunk slots j * kThr + wave * 64 .. + 63 of a tile: tile row
+    // j * kThr / 8 + tid / 8, position tid % 8, which holds chunk (tid % 8) ^ lds_swizzle_key_step2(row). Rows past the
+    // end of the tensor get an offset outside the buffer and read as zero.
     constexpr int kOutside = 0x7FFFFFF0;
-    const int chunk = (tid & 7) ^ lds_swizzle_key_step2(tid >> 3);  // j * 32 does not change the key
-    int voff_a[8], voff_b[8];
+    const int chunk = (tid & 7) ^ lds_swizzle_key_step2(tid >> 3);  // j * kThr / 8 is a multiple of 16: same key
+    int voff_a[kLoads], voff_b[kLoads];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int ra = m0 + j * 32 + (tid >> 3), rb = n0 + j * 32 + (tid >> 3);
+    for (int j = 0; j < kLoads; ++j) {
+        const int ra = m0 + j * (kThr / 8) + (tid >> 3), rb = n0 + j * (kThr / 8) + (tid >> 3);
         voff_a[j] = ra < m ? int(int64_t(ra) * lda) + chunk * 16 : kOutside;
         voff_b[j] = rb < n ? int(int64_t(rb) * ldb) + chunk * 16 : kOutside;
     }
@@ -220,19 +236,19 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
     auto load_a = [&](int step, int slot) {
         uint4 *dst = lds + slot * kTileChunks + wave * 64;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) buffer_load_to_lds_b128(rsrc_a, dst + j * kThreads, voff_a[j], step * kBKB);
+        for (int j = 0; j < kLoads; ++j) buffer_load_to_lds_b128(rsrc_a, dst + j * kThr, voff_a[j], step * kBKB);
     };
     auto load_b = [&](int step, int slot) {
         uint4 *dst = lds + (kASlots + slot) * kTileChunks + wave * 64;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) buffer_load_to_lds_b128(rsrc_b, dst + j * kThreads, voff_b[j], step * kBKB);
+        for (int j = 0; j < kLoads; ++j) buffer_load_to_lds_b128(rsrc_b, dst + j * kThr, voff_b[j], step * kBKB);
     };
 
     // LDS byte addresses of this lane's two 16-byte fragment halves in block 0 of its wave, slot 0 of each ring;
     // block i adds i * 16 rows = i * 2048 bytes
     uint32_t a_addr[2], b_addr[2];
     {
-        const int ra = wm * 128 + ls, rb = wn * 128 + ls;
+        const int ra = wm * 128 + ls, rb = wn * (NB * 16) + ls;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             a_addr[h] = uint32_t((ra * 8 + ((2 * kg + h) ^ lds_swizzle_key_step2(ra))) * 16);
@@ -247,22 +263,20 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
     load_a(1, 1);
     load_b(1, 1);
     load_a(2, 2);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(24));
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(3 * kLoads));
     __builtin_amdgcn_s_barrier();
 
-    int4v_t bf[8][2], af[3][2];
-    // row block i of a step keeps its A fragment in af[i % 3]
+    int4v_t bf[NB][2], af[3][2];
+    // row block i of a step keeps its A fragment in af[i % 3]. First reads in order of first use: b0, a0, b1 ..
     bf[0][0] = lds_read_b128_early<0>(b_addr[0]);
     bf[0][1] = lds_read_b128_early<0>(b_addr[1]);
     af[0][0] = lds_read_b128_early<0>(a_addr[0]);
     af[0][1] = lds_read_b128_early<0>(a_addr[1]);
-    bf[1][0] = lds_read_b128_early<1 * 2048>(b_addr[0]); bf[1][1] = lds_read_b128_early<1 * 2048>(b_addr[1]);
-    bf[2][0] = lds_read_b128_early<2 * 2048>(b_addr[0]); bf[2][1] = lds_read_b128_early<2 * 2048>(b_addr[1]);
-    bf[3][0] = lds_read_b128_early<3 * 2048>(b_addr[0]); bf[3][1] = lds_read_b128_early<3 * 2048>(b_addr[1]);
-    bf[4][0] = lds_read_b128_early<4 * 2048>(b_addr[0]); bf[4][1] = lds_read_b128_early<4 * 2048>(b_addr[1]);
-    bf[5][0] = lds_read_b128_early<5 * 2048>(b_addr[0]); bf[5][1] = lds_read_b128_early<5 * 2048>(b_addr[1]);
-    bf[6][0] = lds_read_b128_early<6 * 2048>(b_addr[0]); bf[6][1] = lds_read_b128_early<6 * 2048>(b_addr[1]);
-    bf[7][0] = lds_read_b128_early<7 * 2048>(b_addr[0]); bf[7][1] = lds_read_b128_early<7 * 2048>(b_addr[1]);
+    static_for<1, NB>([&](auto jt) {
+        constexpr int J = decltype(jt)::value;
+        bf[J][0] = lds_read_b128_early<J * 2048>(b_addr[0]);
+        bf[J][1] = lds_read_b128_early<J * 2048>(b_addr[1]);
+    });
 
     int unit_scales;
     asm volatile("v_mov_b32 %0, 0x7f7f7f7f" : "=v"(unit_scales));
@@ -271,60 +285,40 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
         const uint32_t aa0 = a_addr[0] + uint32_t(a_slot) * kSlotBytes, aa1 = a_addr[1] + uint32_t(a_slot) * kSlotBytes;
         const int a_next = a_slot == kASlots - 1 ? 0 : a_slot + 1, b_next = b_slot ^ 1;
 
-        // ---- row block 0: the reads outstanding are a0, b0 .. b7 of this step (in either order of a0 and b0)
-        lds_wait_keep_newer<14>(bf[0][0], bf[0][1]);
-        lds_wait_keep_newer<14>(af[0][0], af[0][1]);
+        // ---- row block 0: the reads outstanding are a0, b0 .. b(NB-1) of this step (in either order of a0 and b0);
+        // the B fragments arrive one by one, a1 is requested behind the first MFMA
+        lds_wait_keep_newer<2 * (NB - 1)>(bf[0][0], bf[0][1]);
+        lds_wait_keep_newer<2 * (NB - 1)>(af[0][0], af[0][1]);
         mfma_fp8_k128v(bf[0][0], bf[0][1], af[0][0], af[0][1], acc[0][0], unit_scales);
         af[1][0] = lds_read_b128_early<1 * 2048>(aa0);
         af[1][1] = lds_read_b128_early<1 * 2048>(aa1);
-        lds_wait_keep_newer<14>(bf[1][0], bf[1][1]);
-        mfma_fp8_k128v(bf[1][0], bf[1][1], af[0][0], af[0][1], acc[0][1], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_keep_newer<12>(bf[2][0], bf[2][1]);
-        mfma_fp8_k128v(bf[2][0], bf[2][1], af[0][0], af[0][1], acc[0][2], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_keep_newer<10>(bf[3][0], bf[3][1]);
-        mfma_fp8_k128v(bf[3][0], bf[3][1], af[0][0], af[0][1], acc[0][3], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_keep_newer<8>(bf[4][0], bf[4][1]);
-        mfma_fp8_k128v(bf[4][0], bf[4][1], af[0][0], af[0][1], acc[0][4], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_keep_newer<6>(bf[5][0], bf[5][1]);
-        mfma_fp8_k128v(bf[5][0], bf[5][1], af[0][0], af[0][1], acc[0][5], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_keep_newer<4>(bf[6][0], bf[6][1]);
-        mfma_fp8_k128v(bf[6][0], bf[6][1], af[0][0], af[0][1], acc[0][6], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_wait_keep_newer<2>(bf[7][0], bf[7][1]);
-        mfma_fp8_k128v(bf[7][0], bf[7][1], af[0][0], af[0][1], acc[0][7], unit_scales);
-        __builtin_amdgcn_sched_barrier(0);
+        static_for<1, NB>([&](auto jt) {
+            constexpr int J = decltype(jt)::value;
+            lds_wait_keep_newer<2 * (NB - 1 - J) + 2>(bf[J][0], bf[J][1]);
+            mfma_fp8_k128v(bf[J][0], bf[J][1], af[0][0], af[0][1], acc[0][J], unit_scales);
+            __builtin_amdgcn_sched_barrier(0);
+        });
         // barrier P: every wave holds all B fragments of this step, so its B slot can take step s + 2
         __builtin_amdgcn_s_barrier();
         load_b(s + 2, b_slot);
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- row blocks 1 .. 6
-        auto row_block = [&](auto i_tag) {
-            constexpr int I = decltype(i_tag)::value;
+        static_for<1, 7>([&](auto it) {
+            constexpr int I = decltype(it)::value;
             af[(I + 1) % 3][0] = lds_read_b128_early<(I + 1) * 2048>(aa0);
             af[(I + 1) % 3][1] = lds_read_b128_early<(I + 1) * 2048>(aa1);
             lds_wait_keep_newer<2>(af[I % 3][0], af[I % 3][1]);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j], unit_scales);
+            for (int j = 0; j < NB; ++j) mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j], unit_scales);
             __builtin_amdgcn_sched_barrier(0);
-        };
-        row_block(std::integral_constant<int, 1>());
-        row_block(std::integral_constant<int, 2>());
-        row_block(std::integral_constant<int, 3>());
-        row_block(std::integral_constant<int, 4>());
-        row_block(std::integral_constant<int, 5>());
-        row_block(std::integral_constant<int, 6>());
+        });
 
         // ---- row block 7. Barrier L: every wave has read all of this step's A slot, so it can take step s + 3,
-        // and every wave's loads of step s + 1 have landed (the 16 newer ones, A of s + 2 and B of s + 2, may
-        // still be in flight), so the first fragments of step s + 1 can be fetched behind this block's MFMAs.
+        // and every wave's loads of step s + 1 have landed (the newer ones, A of s + 2 and B of s + 2, may still be
+        // in flight), so the first fragments of step s + 1 can be fetched behind this block's MFMAs.
         lds_wait_keep_newer<0>(af[1][0], af[1][1]);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(16));
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * kLoads));
         __builtin_amdgcn_s_barrier();
         load_a(s + 3, a_slot);
         __builtin_amdgcn_sched_barrier(0);
@@ -333,40 +327,29 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
             const uint32_t nb0 = b_addr[0] + uint32_t(b_next) * kSlotBytes, nb1 = b_addr[1] + uint32_t(b_next) * kSlotBytes;
             af[0][0] = lds_read_b128_early<0>(na0);
             af[0][1] = lds_read_b128_early<0>(na1);
-            mfma_fp8_k128v(bf[0][0], bf[0][1], af[1][0], af[1][1], acc[7][0], unit_scales);
-            bf[0][0] = lds_read_b128_early<0 * 2048>(nb0); bf[0][1] = lds_read_b128_early<0 * 2048>(nb1);
-            mfma_fp8_k128v(bf[1][0], bf[1][1], af[1][0], af[1][1], acc[7][1], unit_scales);
-            bf[1][0] = lds_read_b128_early<1 * 2048>(nb0); bf[1][1] = lds_read_b128_early<1 * 2048>(nb1);
-            mfma_fp8_k128v(bf[2][0], bf[2][1], af[1][0], af[1][1], acc[7][2], unit_scales);
-            bf[2][0] = lds_read_b128_early<2 * 2048>(nb0); bf[2][1] = lds_read_b128_early<2 * 2048>(nb1);
-            mfma_fp8_k128v(bf[3][0], bf[3][1], af[1][0], af[1][1], acc[7][3], unit_scales);
-            bf[3][0] = lds_read_b128_early<3 * 2048>(nb0); bf[3][1] = lds_read_b128_early<3 * 2048>(nb1);
-            mfma_fp8_k128v(bf[4][0], bf[4][1], af[1][0], af[1][1], acc[7][4], unit_scales);
-            bf[4][0] = lds_read_b128_early<4 * 2048>(nb0); bf[4][1] = lds_read_b128_early<4 * 2048>(nb1);
-            mfma_fp8_k128v(bf[5][0], bf[5][1], af[1][0], af[1][1], acc[7][5], unit_scales);
-            bf[5][0] = lds_read_b128_early<5 * 2048>(nb0); bf[5][1] = lds_read_b128_early<5 * 2048>(nb1);
-            mfma_fp8_k128v(bf[6][0], bf[6][1], af[1][0], af[1][1], acc[7][6], unit_scales);
-            bf[6][0] = lds_read_b128_early<6 * 2048>(nb0); bf[6][1] = lds_read_b128_early<6 * 2048>(nb1);
-            mfma_fp8_k128v(bf[7][0], bf[7][1], af[1][0], af[1][1], acc[7][7], unit_scales);
-            bf[7][0] = lds_read_b128_early<7 * 2048>(nb0); bf[7][1] = lds_read_b128_early<7 * 2048>(nb1);
+            static_for<0, NB>([&](auto jt) {
+                constexpr int J = decltype(jt)::value;
+                mfma_fp8_k128v(bf[J][0], bf[J][1], af[1][0], af[1][1], acc[7][J], unit_scales);
+                bf[J][0] = lds_read_b128_early<J * 2048>(nb0);
+                bf[J][1] = lds_read_b128_early<J * 2048>(nb1);
+            });
         }
         __builtin_amdgcn_sched_barrier(0);
         a_slot = a_next;
         b_slot = b_next;
     }
     // drain: the look-ahead fragment reads of the step past the end are never used, but their destination
-    // registers must not be reused before they have landed (the wait names every one of them), and LDS must
+    // registers must not be reused before they have landed (the waits name every one of them), and LDS must
     // not be released with tile loads in flight
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(bf[0][0]), "+v"(bf[0][1]), "+v"(bf[1][0]), "+v"(bf[1][1]), "+v"(bf[2][0]), "+v"(bf[2][1]),
-                   "+v"(bf[3][0]), "+v"(bf[3][1]), "+v"(bf[4][0]), "+v"(bf[4][1]), "+v"(bf[5][0]), "+v"(bf[5][1]),
-                   "+v"(bf[6][0]), "+v"(bf[6][1]), "+v"(bf[7][0]), "+v"(bf[7][1]), "+v"(af[0][0]), "+v"(af[0][1]));
+    lds_wait_keep_newer<0>(af[0][0], af[0][1]);
+#pragma unroll
+    for (int j = 0; j < NB; ++j) lds_wait_keep_newer<0>(bf[j][0], bf[j][1]);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     // the compiler does not see the MFMAs inside the asm: let the last ones retire before the accumulators are read
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
-    // acc[i][j][v] = c[m0 + wm*128 + i*16 + ls][n0 + wn*128 + j*16 + 4*kg + v]
+    // acc[i][j][v] = c[m0 + wm*128 + i*16 + ls][n0 + wn*NB*16 + j*16 + 4*kg + v]
     float alpha = 1.0f;
     if (scale_a != nullptr) alpha *= *scale_a;
     if (scale_b != nullptr) alpha *= *scale_b;
@@ -375,8 +358,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_kernel(const uint8_t *__
         const int row = m0 + wm * 128 + i * 16 + ls;
         if (row < m) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int col = n0 + wn * 128 + j * 16 + 4 * kg;
+            for (int j = 0; j < NB; ++j) {
+                const int col = n0 + wn * (NB * 16) + j * 16 + 4 * kg;
                 if (col < n) {  // n % 4 == 0
                     float4_t v = acc[i][j];
 #pragma unroll
@@ -446,21 +429,23 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
         }
         const bool fast = (k % kBKB == 0) && (m - 1) * lda + k <= (int64_t(1) << 30) &&
                           (n - 1) * ldb + k <= (int64_t(1) << 30);
-        // 256 x 256 tiles (4 waves, 160 KiB of LDS) move the fewest bytes per flop and win once they fill the chip twice
-        // over (8192^3: 449 vs 516 us); with fewer tiles the 256 x 128, 8-wave kernel has the better occupancy and tile
-        // granularity (2048 x 4096 x 11008: 102 vs 120 us; 512 x 4096 x 11008: 33 vs 57 us).
-        if (fast && int64_t(tiles_m) * tiles_n < 512) {
-            gemm_fp8_kernel8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
-            return;
-        }
         if (fast) {
+            // 256 x 256 tiles move the fewest bytes per flop; 256 x 128 tiles cost about 15 % more per flop but come in
+            // twice as many pieces. Take whichever needs less time in rounds of one workgroup per CU (measured: 4096^3 60
+            // vs 70 us, 2048 x 4096 x 11008 108 vs 101 us, 1024 x 8192 x 8192 91 vs 65 us).
+            const int64_t t256 = int64_t(tiles_m) * tiles_n, t128 = int64_t(tiles_m) * cdiv(n, 128);
+            const double cost256 = double(cdiv(t256, 256)), cost128 = double(cdiv(t128, 256)) * 0.5 * 1.15;
+            if (cost128 < cost256) {
+                gemm_fp8_kernel8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
+                return;
+            }
             static bool fast_attr_set = false;
             if (!fast_attr_set) {
-                QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_kernel<OUT>),
+                QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_kernel<OUT, 8>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, kFastLdsBytes));
                 fast_attr_set = true;
             }
-            launch(gemm_fp8_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kFastLdsBytes), stream, ap, lda, bp, ldb, c,
+            launch(gemm_fp8_kernel<OUT, 8>, dim3(uint32_t(grid)), dim3(512), size_t(kFastLdsBytes), stream, ap, lda, bp, ldb, c,
                    int(m), int(n), int(k), sa, sb, tiles_m, tiles_n, tiling.xm, tiling.xn);
             return;
         }
