@@ -12,7 +12,10 @@ Pinning status of each function (what independent evidence fixes it):
 
   round_half_away          closed form; tie cases; equals C roundf (checked against the C restatement)
   symmetric_quantize       invariants (scale == amax/qmax bit-for-bit, max|q| == qmax, odd symmetry),
-                           constructed ties, brute force over all f16 patterns, reference test shapes
+                           constructed ties, brute force over all f16 patterns against the reference's own half
+                           type (oracle/_ref where built, and its recorded outputs in tests/golden/ref_half_vectors.npz),
+                           reference test shapes
+  reference_cpu_quant_matmul  bit for bit against the reference's half type (oracle/_ref and the golden vectors)
   symmetric_dequantize     closed form (one multiply); round trip at the reference's tolerance
   symmetric_quant_matmul   reduces to a library matmul on the dequantized weights; exact small-integer cases
   quant_matmul_split_k     sum over parts == full; zero-padded tail part

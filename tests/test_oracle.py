@@ -437,3 +437,40 @@ def test_make_inputs_is_reproducible():
 
 
 _DIGESTS = {'a': '69d00c4eb4c2d624', 'w': 'c64162dabba6a903'}
+
+
+# ----------------------------------------------------------------------------- golden vectors of the reference's half type
+
+def test_oracle_against_golden_vectors_of_reference_half_type():
+    # tests/golden/ref_half_vectors.npz holds operand bit patterns and the results the reference's own CPU half type
+    # (include/hidet/runtime/cpu/float16.h, compiled by oracle/Makefile's `ref` target) produced for them; written by
+    # tests/golden/make_ref_half_vectors.py. This test needs neither the reference checkout nor the built driver.
+    import os
+
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'ref_half_vectors.npz'), allow_pickle=False)
+    fa = g['op_a'].view(np.float16).astype(np.float32)
+    fb = g['op_b'].view(np.float16).astype(np.float32)
+    with np.errstate(over='ignore', divide='ignore', invalid='ignore'):
+        for name, exact in (('mul', fa * fb), ('add', fa + fb), ('div', fa / fb)):
+            # every operator of the type is: widen to float32, operate, round to nearest even
+            assert np.array_equal(exact.astype(np.float32).astype(np.float16).view(np.uint16), g['op_' + name]), name
+    r = O.round_half_away(g['round_in'].view(np.float16).astype(np.float32)).astype(np.float16)
+    assert np.array_equal(r.view(np.uint16), g['round_out'])
+    with np.errstate(over='ignore'):
+        assert np.array_equal(g['cvt_f32'].astype(np.float16).view(np.uint16), g['cvt_f16'])
+        L = clib.lib()
+        ours = np.array([L.oracle_f32_to_f16(float(x)) for x in g['cvt_f32']], dtype=np.uint16)  # the C restatement's own conversion
+        assert np.array_equal(ours, g['cvt_f16'])
+    # symmetric_quantize on float16 columns, every operator in the reference's half arithmetic. The oracle saturates
+    # where the reference's cast wraps (a quotient that rounds to 128): those codes read -128 in the fixture.
+    w16 = g['quant_w_bits'].view(np.float16)
+    q, s = O.symmetric_quantize(w16, 'int8', dims=0)
+    assert np.array_equal(s.view(np.uint16), g['quant_scale_bits'])
+    differs = q != g['quant_codes']
+    assert np.all(g['quant_codes'][differs] == -128) and np.all(q[differs] == 127) and differs.sum() <= 4
+    # the reference's CPU route of the matmul (float16 accumulator), restated in numpy and in C
+    a = g['mm_a_bits'].view(np.float16)
+    sc = g['mm_scale_bits'].view(np.float16)
+    want = g['mm_c_bits'].view(np.float16)
+    assert np.array_equal(O.reference_cpu_quant_matmul(a, g['mm_w'], sc).view(np.uint16), g['mm_c_bits'])
+    assert np.array_equal(clib.quant_matmul_ref_cpu(a, g['mm_w'], sc).view(np.uint16), want.view(np.uint16))
