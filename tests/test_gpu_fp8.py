@@ -49,7 +49,9 @@ def test_quantize_per_tensor_bit_exact():
 
 @pytest.mark.parametrize('a_shape, b_shape', [[[256, 128], [256, 128]], [[4096, 4096], [4096, 4096]], [[512, 256], [128, 256]],
                                               [[1, 256], [48, 256]], [[16, 1024], [200, 1024]], [[100, 48], [36, 48]],
-                                              [[300, 272], [260, 272]]])
+                                              [[300, 272], [260, 272]],
+                                              # 512 tiles of 256 x 256 (two rounds of workgroups), 2 and 1 k-steps each; ragged edges
+                                              [[4096, 256], [8192, 256]], [[4096, 128], [8192, 128]], [[4000, 384], [8100, 384]]])
 def test_matmul_f8_reference_recipe(a_shape, b_shape):
     # tests/operators_core/test_matmul.py:250-288: randint(-3, 3) inputs; the exact integer result is the answer
     announce('matmul_f8', a_shape, b_shape)
