@@ -92,6 +92,65 @@ __global__ __launch_bounds__(256) void quantize_kernel(const void *__restrict__ 
     store_code<QT>(q, i, code);
 }
 
+// Same arithmetic, four consecutive elements of the innermost axis per thread (inner a multiple of 4, tensors aligned
+// for the 4-element accesses): one index division per four elements, 16- or 8-byte loads, 4- or 8-byte code stores.
+// ALONG_REDUCE (inner == 1, reduce a multiple of 4): the four elements lie along the reduced axis and share one scale;
+// R is then reduce / 4 and inner4 is unused.
+template <int DT, int QT, bool ALONG_REDUCE>
+__global__ __launch_bounds__(256) void quantize4_kernel(const void *__restrict__ w, const uint32_t *__restrict__ amax_bits,
+                                                        void *__restrict__ q, void *__restrict__ scale, int64_t R,
+                                                        int64_t inner4, int64_t total4) {
+    const float qmax = QT == HIDET_QMM_I8 ? 127.0f : 32767.0f;
+    const int64_t i4 = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i4 >= total4) return;
+    int64_t r, sidx;
+    uint32_t abits[4];
+    if (ALONG_REDUCE) {
+        sidx = i4 / R;
+        r = i4 - sidx * R;
+        abits[0] = abits[1] = abits[2] = abits[3] = amax_bits[sidx];
+    } else {
+        const int64_t row = i4 / inner4;  // o * R + r
+        const int64_t c4 = i4 - row * inner4;
+        const int64_t o = row / R;
+        r = row - o * R;
+        sidx = (o * inner4 + c4) * 4;
+        const uint4 ab = *reinterpret_cast<const uint4 *>(amax_bits + sidx);
+        abits[0] = ab.x; abits[1] = ab.y; abits[2] = ab.z; abits[3] = ab.w;
+    }
+    float x[4];
+    if (DT == HIDET_QMM_F32) {
+        const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(w) + i4 * 4);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(w) + i4 * 4);
+        const uint16_t h[4] = {uint16_t(v.x), uint16_t(v.x >> 16), uint16_t(v.y), uint16_t(v.y >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = DT == HIDET_QMM_F16 ? f16_bits_to_f32(h[e]) : bf16_bits_to_f32(h[e]);
+    }
+    float code[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float s = round_to<DT>(__uint_as_float(abits[e]) / qmax);
+        if (r == 0 && (!ALONG_REDUCE || e == 0)) store_from_f32<DT>(scale, sidx + (ALONG_REDUCE ? 0 : e), s);
+        code[e] = s != 0.0f ? roundf(round_to<DT>(x[e] / s)) : 0.0f;
+    }
+    if (QT == HIDET_QMM_I8) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) packed |= uint32_t(uint8_t(int8_t(fminf(fmaxf(code[e], -128.0f), 127.0f)))) << (8 * e);
+        static_cast<uint32_t *>(q)[i4] = packed;
+    } else {
+        uint2 packed;
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = uint32_t(uint16_t(int16_t(fminf(fmaxf(code[e], -32768.0f), 32767.0f))));
+        packed.x = h[0] | (h[1] << 16);
+        packed.y = h[2] | (h[3] << 16);
+        static_cast<uint2 *>(q)[i4] = packed;
+    }
+}
+
 template <int QT, int ST>
 __global__ __launch_bounds__(256) void dequantize_kernel(const void *__restrict__ q, const void *__restrict__ scale,
                                                          void *__restrict__ w, int64_t R, int64_t inner, int64_t total) {
@@ -219,6 +278,26 @@ HIDET_API void hidet_symmetric_quantize(const void *w, void *wq, void *scale, in
                    inner, rows_per_split, int(splits > 1));
         }
         if (total == 0) return;
+        const int esize = DT == HIDET_QMM_F32 ? 4 : 2, qsize = q_dtype == HIDET_QMM_I8 ? 1 : 2;
+        const bool vec_ok = aligned(w, 4 * esize) && aligned(wq, 4 * qsize) && aligned(scale, esize);
+        if (vec_ok && inner % 4 == 0) {
+            if (q_dtype == HIDET_QMM_I8)
+                launch(quantize4_kernel<DT, HIDET_QMM_I8, false>, dim3(cdiv(total / 4, 256)), dim3(256), 0, stream, w, amax_bits,
+                       wq, scale, reduce, inner / 4, total / 4);
+            else
+                launch(quantize4_kernel<DT, HIDET_QMM_I16, false>, dim3(cdiv(total / 4, 256)), dim3(256), 0, stream, w, amax_bits,
+                       wq, scale, reduce, inner / 4, total / 4);
+            return;
+        }
+        if (vec_ok && inner == 1 && reduce % 4 == 0) {
+            if (q_dtype == HIDET_QMM_I8)
+                launch(quantize4_kernel<DT, HIDET_QMM_I8, true>, dim3(cdiv(total / 4, 256)), dim3(256), 0, stream, w, amax_bits,
+                       wq, scale, reduce / 4, int64_t(0), total / 4);
+            else
+                launch(quantize4_kernel<DT, HIDET_QMM_I16, true>, dim3(cdiv(total / 4, 256)), dim3(256), 0, stream, w, amax_bits,
+                       wq, scale, reduce / 4, int64_t(0), total / 4);
+            return;
+        }
         if (q_dtype == HIDET_QMM_I8)
             launch(quantize_kernel<DT, HIDET_QMM_I8>, dim3(cdiv(total, 256)), dim3(256), 0, stream, w, amax_bits, wq, scale,
                    reduce, inner, total);
