@@ -229,6 +229,61 @@ __global__ __launch_bounds__(256) void fp8_quantize_kernel(const void *__restric
     codes[i] = s == 0.0f ? uint8_t(0) : f32_to_e4m3(load_as_f32<DT>(x, i) / s);
 }
 
+// Four-element forms (numel a multiple of 4, 16-byte aligned input, 4-byte aligned codes).
+template <int DT>
+__device__ __forceinline__ void load4_as_f32(const void *p, int64_t i4, float (&x)[4]) {
+    if (DT == HIDET_QMM_F32) {
+        const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(p) + i4 * 4);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(p) + i4 * 4);
+        const uint16_t h[4] = {uint16_t(v.x), uint16_t(v.x >> 16), uint16_t(v.y), uint16_t(v.y >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = DT == HIDET_QMM_F16 ? f16_bits_to_f32(h[e]) : bf16_bits_to_f32(h[e]);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void amax_all4_kernel(const void *__restrict__ x, uint32_t *__restrict__ amax_bits, int64_t numel4) {
+    __shared__ float red[4];
+    float m = 0.0f;
+    for (int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x; i < numel4; i += int64_t(gridDim.x) * 256) {
+        float v[4];
+        load4_as_f32<DT>(x, i, v);
+        m = fmaxf(fmaxf(m, fmaxf(fabsf(v[0]), fabsf(v[1]))), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        atomicMax(amax_bits, __float_as_uint(m));
+    }
+}
+
+// The quotient is clamped to +-448 (what saturation means for a format whose largest finite value is 448) and converted
+// by the hardware's round-to-nearest-even OCP e4m3 conversion, two values per instruction.
+template <int DT>
+__global__ __launch_bounds__(256) void fp8_quantize4_kernel(const void *__restrict__ x, const uint32_t *__restrict__ amax_bits,
+                                                            uint32_t *__restrict__ codes, float *__restrict__ scale, int64_t numel4) {
+    const float s = __uint_as_float(*amax_bits) / 448.0f;
+    const int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i == 0) *scale = s;
+    if (i >= numel4) return;
+    float v[4];
+    load4_as_f32<DT>(x, i, v);
+    uint32_t packed = 0;
+    if (s != 0.0f) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = fminf(fmaxf(v[e] / s, -448.0f), 448.0f);
+        int p = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+        p = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], p, true);
+        packed = uint32_t(p);
+    }
+    codes[i] = packed;
+}
+
 template <typename F>
 void dispatch_float(int dt, F &&f) {
     switch (dt) {
@@ -364,6 +419,14 @@ HIDET_API void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *s
     launch_aux(fill_u32_kernel, dim3(1), dim3(64), 0, stream, amax_bits, int64_t(1), 0u);
     dispatch_float(x_dtype, [&](auto dt) {
         constexpr int DT = decltype(dt)::value;
+        const int esize = DT == HIDET_QMM_F32 ? 4 : 2;
+        if (numel > 0 && numel % 4 == 0 && aligned(x, 4 * esize) && aligned(codes, 4)) {
+            const int64_t n4 = numel / 4;
+            launch(amax_all4_kernel<DT>, dim3(std::min<int64_t>(cdiv(n4, 256 * 4), 4096)), dim3(256), 0, stream, x, amax_bits, n4);
+            launch(fp8_quantize4_kernel<DT>, dim3(cdiv(n4, 256)), dim3(256), 0, stream, x, amax_bits,
+                   static_cast<uint32_t *>(codes), static_cast<float *>(scale), n4);
+            return;
+        }
         if (numel > 0) {
             const int64_t blocks = std::min<int64_t>(cdiv(numel, 256 * 8), 2048);
             launch(amax_all_kernel<DT>, dim3(blocks), dim3(256), 0, stream, x, amax_bits, numel);

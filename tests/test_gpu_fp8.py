@@ -47,6 +47,23 @@ def test_quantize_per_tensor_bit_exact():
     assert zs.item() == 0 and not codes_of(z).any()
 
 
+def test_quantize_per_tensor_every_rounding_boundary():
+    # amax = 448 makes the scale exactly 1, so the codes are e4m3(x): every midpoint between two neighbouring e4m3 values
+    # and its two float32 neighbours, both signs, plus the values themselves. The fast kernel converts in hardware, the
+    # oracle in integer arithmetic; ties must go to even in both.
+    announce('fp8 quantize rounding boundaries')
+    vals = O.e4m3_decode(np.arange(0, 0x7F, dtype=np.uint8)).astype(np.float32)      # 0 .. 448, ascending
+    mids = ((vals[:-1].astype(np.float64) + vals[1:].astype(np.float64)) / 2).astype(np.float32)
+    pts = np.concatenate([vals, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)),
+                          np.array([2.0 ** -10, 2.0 ** -10 * 0.99, 2.0 ** -11, 1e-12, 447.99, 440.0], dtype=np.float32)])
+    pts = np.concatenate([pts, -pts]).astype(np.float32)
+    pts = np.concatenate([pts, np.zeros((-pts.size) % 4, dtype=np.float32)])          # multiple of 4: the vector kernel
+    for x in (pts, pts[:-1]):                                                         # ... and the scalar one
+        codes, scale = F8.fp8_quantize_per_tensor(dev(x))
+        assert scale.item() == 1.0
+        assert np.array_equal(codes_of(codes), O.e4m3_encode(x))
+
+
 @pytest.mark.parametrize('a_shape, b_shape', [[[256, 128], [256, 128]], [[4096, 4096], [4096, 4096]], [[512, 256], [128, 256]],
                                               [[1, 256], [48, 256]], [[16, 1024], [200, 1024]], [[100, 48], [36, 48]],
                                               [[300, 272], [260, 272]],
