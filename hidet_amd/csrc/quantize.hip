@@ -73,6 +73,20 @@ __device__ __forceinline__ void store_code(void *q, int64_t i, float r) {
     }
 }
 
+// Four-element forms (numel a multiple of 4, 16-byte aligned input, 4-byte aligned codes).
+template <int DT>
+__device__ __forceinline__ void load4_as_f32(const void *p, int64_t i4, float (&x)[4]) {
+    if (DT == HIDET_QMM_F32) {
+        const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(p) + i4 * 4);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else {
+        const uint2 v = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(p) + i4 * 4);
+        const uint16_t h[4] = {uint16_t(v.x), uint16_t(v.x >> 16), uint16_t(v.y), uint16_t(v.y >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = DT == HIDET_QMM_F16 ? f16_bits_to_f32(h[e]) : bf16_bits_to_f32(h[e]);
+    }
+}
+
 // code = saturating_cast(round_half_away(rnd(w / scale))), scale = rnd(amax / qmax), rnd = round to w's dtype.
 template <int DT, int QT>
 __global__ __launch_bounds__(256) void quantize_kernel(const void *__restrict__ w, const uint32_t *__restrict__ amax_bits,
@@ -162,6 +176,43 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const void *__restrict_
     store_from_f32<ST>(w, i, round_to<ST>(code * load_as_f32<ST>(scale, o * inner + c)));
 }
 
+// Four consecutive elements per thread: along the innermost axis (inner4 = inner / 4, one scale each) or, with
+// ALONG_REDUCE (inner == 1, R = reduce / 4), along the reduced axis (one scale for all four).
+template <int QT, int ST, bool ALONG_REDUCE>
+__global__ __launch_bounds__(256) void dequantize4_kernel(const void *__restrict__ q, const void *__restrict__ scale,
+                                                          void *__restrict__ w, int64_t R, int64_t inner4, int64_t total4) {
+    const int64_t i4 = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i4 >= total4) return;
+    float code[4], sc[4];
+    if (QT == HIDET_QMM_I8) {
+        const uint32_t v = static_cast<const uint32_t *>(q)[i4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) code[e] = float(int8_t(v >> (8 * e)));
+    } else {
+        const uint2 v = static_cast<const uint2 *>(q)[i4];
+        code[0] = float(int16_t(v.x)); code[1] = float(int16_t(v.x >> 16));
+        code[2] = float(int16_t(v.y)); code[3] = float(int16_t(v.y >> 16));
+    }
+    if (ALONG_REDUCE) {
+        sc[0] = sc[1] = sc[2] = sc[3] = load_as_f32<ST>(scale, i4 / R);
+    } else {
+        const int64_t row = i4 / inner4;
+        const int64_t sidx = ((row / R) * inner4 + (i4 - row * inner4)) * 4;
+        load4_as_f32<ST>(scale, sidx / 4, sc);
+    }
+    float out[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = round_to<ST>(code[e] * sc[e]);
+    if (ST == HIDET_QMM_F32) {
+        static_cast<float4 *>(w)[i4] = float4{out[0], out[1], out[2], out[3]};
+    } else {
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h[e] = ST == HIDET_QMM_F16 ? f32_to_f16_bits(out[e]) : f32_to_bf16_bits(out[e]);
+        static_cast<uint2 *>(w)[i4] = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+    }
+}
+
 // Group-wise int4: grid (ceil(n/128), k/group); 256 threads = 4 row lanes x 64 column pairs.
 // scale32 = amax / 7 and code = clamp(round_half_away(w / scale32), -7, 7) in float32; two codes per
 // byte along n, low nibble first; the stored scale is scale32 rounded to the scale dtype.
@@ -227,20 +278,6 @@ __global__ __launch_bounds__(256) void fp8_quantize_kernel(const void *__restric
     if (i == 0) *scale = s;
     if (i >= numel) return;
     codes[i] = s == 0.0f ? uint8_t(0) : f32_to_e4m3(load_as_f32<DT>(x, i) / s);
-}
-
-// Four-element forms (numel a multiple of 4, 16-byte aligned input, 4-byte aligned codes).
-template <int DT>
-__device__ __forceinline__ void load4_as_f32(const void *p, int64_t i4, float (&x)[4]) {
-    if (DT == HIDET_QMM_F32) {
-        const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(p) + i4 * 4);
-        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-    } else {
-        const uint2 v = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(p) + i4 * 4);
-        const uint16_t h[4] = {uint16_t(v.x), uint16_t(v.x >> 16), uint16_t(v.y), uint16_t(v.y >> 16)};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[e] = DT == HIDET_QMM_F16 ? f16_bits_to_f32(h[e]) : bf16_bits_to_f32(h[e]);
-    }
 }
 
 template <int DT>
@@ -381,6 +418,21 @@ HIDET_API void hidet_symmetric_dequantize(const void *wq, const void *scale, voi
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     dispatch_float(s_dtype, [&](auto dt) {
         constexpr int ST = decltype(dt)::value;
+        const int esize = ST == HIDET_QMM_F32 ? 4 : 2, qsize = q_dtype == HIDET_QMM_I8 ? 1 : 2;
+        const bool vec_ok = aligned(w, 4 * esize) && aligned(wq, 4 * qsize) && aligned(scale, 4 * esize);
+        auto go4 = [&](auto kern, int64_t r4, int64_t in4) {
+            launch(kern, dim3(cdiv(total / 4, 256)), dim3(256), 0, stream, wq, scale, w, r4, in4, total / 4);
+        };
+        if (vec_ok && inner % 4 == 0) {
+            if (q_dtype == HIDET_QMM_I8) go4(dequantize4_kernel<HIDET_QMM_I8, ST, false>, reduce, inner / 4);
+            else go4(dequantize4_kernel<HIDET_QMM_I16, ST, false>, reduce, inner / 4);
+            return;
+        }
+        if (vec_ok && inner == 1 && reduce % 4 == 0) {
+            if (q_dtype == HIDET_QMM_I8) go4(dequantize4_kernel<HIDET_QMM_I8, ST, true>, reduce / 4, int64_t(0));
+            else go4(dequantize4_kernel<HIDET_QMM_I16, ST, true>, reduce / 4, int64_t(0));
+            return;
+        }
         if (q_dtype == HIDET_QMM_I8)
             launch(dequantize_kernel<HIDET_QMM_I8, ST>, dim3(cdiv(total, 256)), dim3(256), 0, stream, wq, scale, w, reduce, inner, total);
         else
