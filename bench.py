@@ -13,6 +13,7 @@ The same JSON line carries
                 bounded sample of the same workload;
   prefill       the M = 2048 GEMM of the same weight shape as TFLOP/s (second half of the metric);
   fp8_prefill   the e4m3 GEMM [4096, 8192] x [8192, 8192]^T -> bf16 with per-tensor scales as TFLOP/s;
+  other_configs one duration / throughput / roofline fraction for each remaining benchmark configuration;
   parity        max relative error of one ring entry against the oracle.
 """
 import argparse
@@ -248,6 +249,71 @@ def main():
     fd = np.array(fd[4:])
     fp8_tflops = 2.0 * MF * KF * NF / (fd.mean() * 1e-6) / 1e12
 
+    # ---- the other benchmark configurations, one figure each (kernel duration through the timing hook, distinct weight
+    # buffers per launch so that nothing is served from the last-level cache) ------------------------------------------
+    def time_kernel(fn, reps, skip):
+        e0, e1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
+        d = []
+        for rep in range(reps):
+            lib.hidet_qmm_arm_timing(e0, e1)
+            fn(rep)
+            lib.hidet_qmm_event_synchronize(e1)
+            d.append(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3)
+        lib.hidet_qmm_event_destroy(e0)
+        lib.hidet_qmm_event_destroy(e1)
+        return float(np.mean(d[skip:]))
+
+    def hbm_entry(us, nbytes):
+        return {'kernel_us': round(us, 2), 'GB/s': round(nbytes / us / 1e3, 1), 'frac_of_hbm_peak': round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    def mfma_entry(us, flops, peak):
+        return {'kernel_us': round(us, 2), 'TFLOP/s': round(flops / us / 1e6, 1), 'frac_of_mfma_peak': round(flops / us / 1e6 / peak, 4)}
+
+    others = {}
+    # W8A16, M = 16, 4096 x 4096 (the reference's CPU-runnable case)
+    w16 = [torch.randint(-127, 128, (4096, 4096), device=device, dtype=torch.int8) for _ in range(32)]  # 2 x the 256 MB LLC
+    s16 = ss[0][:4096].contiguous()
+    a16 = torch.randn((16, 4096), generator=g, device=device, dtype=torch.float32).to(torch.float16)
+    c16 = torch.empty((16, 4096), dtype=torch.float16, device=device)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', a16, w16[r % 32], s16, c16, 16, 4096, 4096, 4096, 0,
+                                      work, work.numel(), sptr), 96, 32)
+    others['w8a16_m16_k4096_n4096'] = hbm_entry(us, 4096 * 4096 + 2 * 4096 + 2 * 16 * 4096 * 2)
+    del w16
+    # W8A16 decode GEMV, down-proj shape [1, 11008] x [11008, 4096]: the ring's buffers reinterpreted as [11008, 4096]
+    ad = torch.randn((1, N), generator=g, device=device, dtype=torch.float32).to(torch.float16)
+    cd = torch.empty((1, K), dtype=torch.float16, device=device)
+    sd = ss[0][:K].contiguous()
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ad, ws[r % RING].view(N, K), sd, cd, 1, N, K, N, 0,
+                                      work, work.numel(), sptr), 48, 16)
+    others['w8a16_gemv_down_proj_k11008_n4096'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * K)
+    # W8A16 prefill, attention QKV shape [2048, 4096] x [4096, 12288]
+    wq = [torch.randint(-127, 128, (K, 12288), device=device, dtype=torch.int8) for _ in range(4)]
+    sq = torch.cat([ss[0], ss[1]])[:12288].contiguous()
+    cq = torch.empty((MP, 12288), dtype=torch.float16, device=device)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ap, wq[r % 4], sq, cq, MP, K, 12288, K, 0, work,
+                                      work.numel(), sptr), 16, 4)
+    others['w8a16_prefill_m2048_k4096_n12288'] = mfma_entry(us, 2.0 * MP * K * 12288, MFMA_F16_PEAK_TFLOPS)
+    del wq, cq
+    # group-wise W4A16 (bf16, group 128), M in {1, 16, 512}
+    w4 = [torch.randint(0, 256, (K, N // 2), device=device, dtype=torch.uint8) for _ in range(16)]
+    s4 = (torch.rand((K // 128, N), generator=g, device=device) * 0.01 + 0.001).to(torch.bfloat16)
+    for m4 in (1, 16, 512):
+        a4 = torch.randn((m4, K), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+        c4 = torch.empty((m4, N), dtype=torch.bfloat16, device=device)
+        us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16', a4, w4[r % 16], s4, c4, m4, K, N, K, 128, 2, 0,
+                                          work, work.numel(), sptr), 40, 16)
+        nbytes = K * N // 2 + 2 * (K // 128) * N + 2 * m4 * K + 2 * m4 * N
+        others['w4a16_m{}_k4096_n11008'.format(m4)] = (hbm_entry(us, nbytes) if m4 <= 16 else
+                                                      mfma_entry(us, 2.0 * m4 * K * N, MFMA_F16_PEAK_TFLOPS))
+    del w4
+    # FP8 decode variant: M = 1 against the same b
+    a1 = a8[:1].contiguous()
+    c1 = torch.empty((1, NF), dtype=torch.bfloat16, device=device)
+    bring = [bq for bq, _ in b8s] + [torch.randint(0, 0x7F, (NF, KF), device=device, dtype=torch.uint8) for _ in range(5)]  # 8 x 64 MiB
+    us = time_kernel(lambda r: ffi.call('hidet_matmul_f8', a1, bring[r % 8], c1, 1, NF, KF, KF, KF, 2, sa, b8s[0][1], sptr), 32, 8)
+    del bring
+    others['fp8_gemv_m1_k8192_n8192'] = hbm_entry(us, NF * KF + KF + 2 * NF + 8)
+
     if args.data_dependence:
         def timed(fn, reps=24):
             e0, e1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
@@ -297,6 +363,7 @@ def main():
                         'roofline': {'bound': 'mfma', 'achieved': round(fp8_tflops, 1), 'peak': MFMA_FP8_PEAK_TFLOPS,
                                      'unit': 'TFLOP/s', 'frac': round(fp8_tflops / MFMA_FP8_PEAK_TFLOPS, 4)},
                         'max_rel_err_vs_oracle_rows_sample': fp8_parity, 'tolerance': 3e-2},
+        'other_configs': others,
         'parity': {'max_rel_err_vs_oracle': parity, 'tolerance': 1e-2, 'graph_replay_matches_eager': replay_ok},
     }
     if not args.no_cpu_baseline:
