@@ -105,29 +105,51 @@ __device__ __forceinline__ void skinny_reduce_store(const float4_t (&res)[16], i
                 for (int u = 0; u < 16; ++u) v += part[u];
             }
             c[col] = skinny_to_out<OutT>(v * s);
-        } else {
-            // rows in groups of 4, splits in groups of 4: 16 loads in flight, each row added in split order
-            for (int row0 = 0; row0 < m; row0 += 4) {
-                float v[4] = {0.f, 0.f, 0.f, 0.f};
-                for (int sp0 = 0; sp0 < splits; sp0 += 4) {
-                    float part[4][4];
+        }
+    }
+    if (m > 1) {
+        // 256 threads = 4 row lanes x 64 column quads: thread (rl, cq) sums rows rl, rl + 4, ... of columns 4cq .. 4cq+3
+        // with 16-byte agent-scope loads, two rows x eight splits = 16 loads in flight, each row added in split order.
+        const int cq = tid & 63, rl = tid >> 6;
+        const int col4 = tile * kSkinnyTileN + cq * 4;
+        if (col4 < n) {  // n is a multiple of 16 on this path: the quad is in or out as a whole
+            constexpr int kAgentScope = 1 << 4;  // sc1
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                partials + int64_t(tile) * splits * m * kSkinnyTileN, 0, splits * m * kSkinnyTileN * 4, 0x00020000);
+            float s4[4] = {1.f, 1.f, 1.f, 1.f};
+            if (col_scale != nullptr) {
 #pragma unroll
-                    for (int u = 0; u < 4; ++u)
+                for (int e = 0; e < 4; ++e) s4[e] = float(col_scale[col4 + e]);
+            }
+            for (int row0 = rl; row0 < m; row0 += 8) {
+                float4_t v[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
+                for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+                    uint4v_t part[2][8];
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            part[u][r] = 0.f;
-                            if (sp0 + u < splits && row0 + r < m)
-                                part[u][r] = __hip_atomic_load(base + (int64_t(sp0 + u) * m + row0 + r) * kSkinnyTileN + tid,
-                                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int r = 0; r < 2; ++r)
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) {
+                            const int row = row0 + 4 * r, sp = sp0 + u;
+                            // past the last row or split: an offset outside the buffer, which reads as zero
+                            const int off = (row < m && sp < splits) ? ((sp * m + row) * kSkinnyTileN + cq * 4) * 4 : 0x7FFFFFF0;
+                            part[r][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAgentScope);
                         }
 #pragma unroll
-                    for (int u = 0; u < 4; ++u)
+                    for (int r = 0; r < 2; ++r)
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) v[r] += part[u][r];
+                        for (int u = 0; u < 8; ++u) v[r] += __builtin_bit_cast(float4_t, part[r][u]);
                 }
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    if (row0 + r < m) c[int64_t(row0 + r) * n + col] = skinny_to_out<OutT>(v[r] * s);
+                for (int r = 0; r < 2; ++r) {
+                    const int row = row0 + 4 * r;
+                    if (row < m) {
+                        uint16_t h[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, skinny_to_out<OutT>(v[r][e] * s4[e]));
+                        *reinterpret_cast<uint2 *>(c + int64_t(row) * n + col4) =
+                            uint2{uint32_t(h[0]) | (uint32_t(h[1]) << 16), uint32_t(h[2]) | (uint32_t(h[3]) << 16)};
+                    }
+                }
             }
         }
     }

@@ -202,7 +202,7 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     const uint8_t *wp = static_cast<const uint8_t *>(w);
     const uint16_t *sp = static_cast<const uint16_t *>(scales);
     uint16_t *cp0 = static_cast<uint16_t *>(c);
-    if (!skinny_w4a16_fast(w, scales, k, n, group)) {
+    if (!skinny_w4a16_fast(w, scales, k, n, group) || !aligned(c, 8)) {  // 8-byte output stores in the split-K sum
         if (dtype == HIDET_QMM_F16)
             launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
         else

@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void naive_w8a16_kernel(const _Float16 *__rest
 
 void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                          int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
-    const bool fast = (n % 16 == 0) && aligned(w, 16) && k > 0;
+    const bool fast = (n % 16 == 0) && aligned(w, 16) && aligned(c, 8) && k > 0;  // 8-byte output stores in the split-K sum
     if (!fast) {
         launch(naive_w8a16_kernel, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, static_cast<const _Float16 *>(a), lda,
                static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(c), m, k, n);
