@@ -160,20 +160,28 @@ __device__ __forceinline__ bool gemm_work_item(int tiles_m, int tiles_n, int xm,
 // waits for the writes to be acknowledged and counts itself in; the part that arrives last reads all of them back
 // in part order - so the sum does not depend on arrival order - and returns true with the sums in `acc`: it finishes
 // the tile. The others return false. The counter goes back to zero for the next launch. `flag` is one int of LDS.
+// Bit r of `rows_valid` says whether acc[r][*] holds rows inside the matrix: the others are exchanged at an offset
+// past the end of the buffer, where the hardware drops stores and answers loads with zero without touching memory,
+// which keeps the exchange of a short matrix (few valid rows in a tall tile) short. (Branching around them instead
+// costs the GEMM kernels registers they do not have.)
 template <int THREADS, int R, int T>
 __device__ __forceinline__ bool gemm_k_split_fixup(float4_t (&acc)[R][T], const GemmWorkItem &item,
-                                                   float *__restrict__ partials, uint32_t *__restrict__ counters, int *flag) {
+                                                   float *__restrict__ partials, uint32_t *__restrict__ counters, int *flag,
+                                                   uint32_t rows_valid) {
     constexpr int kTileFloats = THREADS * R * T * 4;
     constexpr int kAgentScope = 1 << 4;  // sc1
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
         partials + int64_t(item.slot) * item.parts * kTileFloats, 0, item.parts * kTileFloats * 4, 0x00020000);
     const int lane_off = threadIdx.x * 16;
+    constexpr int kOutside = 0x7FFFFFF0;  // past the end of the buffer: the store is dropped, the load returns zero
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+    for (int r = 0; r < R; ++r) {
+        const int off = ((rows_valid >> r) & 1u) ? lane_off : kOutside;
 #pragma unroll
         for (int t = 0; t < T; ++t)
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v_t, acc[r][t]), rsrc, lane_off,
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v_t, acc[r][t]), rsrc, off,
                                                    ((item.part * R + r) * T + t) * (THREADS * 16), kAgentScope);
+    }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // vmcnt(0): every store of this lane has been acknowledged
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -190,10 +198,11 @@ __device__ __forceinline__ bool gemm_k_split_fixup(float4_t (&acc)[R][T], const 
     for (int p = 0; p < item.parts; ++p) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
+            const int off = ((rows_valid >> r) & 1u) ? lane_off : kOutside;
             uint4v_t v[T];
 #pragma unroll
             for (int t = 0; t < T; ++t)
-                v[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, ((p * R + r) * T + t) * (THREADS * 16), kAgentScope);
+                v[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, ((p * R + r) * T + t) * (THREADS * 16), kAgentScope);
 #pragma unroll
             for (int t = 0; t < T; ++t) acc[r][t] += __builtin_bit_cast(float4_t, v[t]);
         }

@@ -1,7 +1,7 @@
 // Group-wise W4A16 GEMM (M > 32): c[m, n] = sum_g scale[g, n] * sum_{k in g} a[m, k] * q[k, n] on
 // bf16 / fp16 MFMA with fp32 accumulation.
 //
-// As in the int8 GEMM the packed weights go straight from global memory into registers: lane (kg, ns)
+// In the register kernels the packed weights go straight from global memory into registers: lane (kg, ns)
 // loads one dword (8 columns) of rows 8kg .. 8kg+7 per 32-row k-step, a wave covers 128 columns.  Each
 // nibble is dequantised exactly as the definition says: u = nibble ^ 8 = q + 8 is widened with
 // v_cvt_f32_ubyte, one fma gives q * scale = u * scale - 8 * scale in fp32 and v_cvt_pk rounds two
@@ -9,12 +9,15 @@
 // values of one column over eight rows are the B operand of a 16x16x32 MFMA.  A wave owns RB*16 rows
 // x 128 columns.
 //
-// Two kernels.  gemm_w4a16_kernel16 (K a multiple of 64, group size a multiple of 64, tensors addressable with 31-bit
-// offsets) is built like the int8 GEMM: buffer loads without address arithmetic, the activation tile straight into
-// a three-slot LDS ring (buffer_load ... lds) two stages ahead, the A fragments of a k-step read one k-step ahead by
-// hand-placed ds_read_b128, the raw weight rows of a k-step refilled one stage ahead as soon as they are consumed, the
-// group's scales fetched one stage before the group starts, 2D XCD regions and the deterministic K split for grids that
-// leave CUs idle.  gemm_w4a16_kernel (register-staged, double-buffered LDS, every load predicated) takes the rest.
+// Three kernels.  gemm_w4a16_lds_kernel (K and group size multiples of 64, N a multiple of 32, tensors addressable
+// with 31-bit offsets) widens each weight once per workgroup into an LDS tile and is described where it is defined.
+// gemm_w4a16_kernel16 (same conditions without the one on N; used where 256-row tiles fit the matrix badly) is built
+// like the int8 GEMM and widens in registers as described above: buffer loads without address arithmetic, the
+// activation tile straight into a three-slot LDS ring (buffer_load ... lds) two stages ahead, the A fragments of a
+// k-step read one k-step ahead by hand-placed ds_read_b128, the raw weight rows of a k-step refilled one stage ahead
+// as soon as they are consumed, the group's scales fetched one stage before the group starts.  Both use 2D XCD
+// regions and the deterministic K split for grids that leave CUs idle.  gemm_w4a16_kernel (register-staged,
+// double-buffered LDS, every load predicated) takes the rest.
 #include "common.h"
 #include "gemm_tiling.h"
 
@@ -417,7 +420,12 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w4a16_kernel16(
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __builtin_amdgcn_sched_barrier(0);
 
-    if (item.parts > 1 && !gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last)) return;
+    if (item.parts > 1) {
+        uint32_t rows_valid = 0;  // row blocks of this wave that reach into the matrix
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) rows_valid |= uint32_t(m0 + (wm * RB + rb) * 16 < m) << rb;
+        if (!gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last, rows_valid)) return;
+    }
 
     if (!col_ok) return;
 #pragma unroll
@@ -465,6 +473,376 @@ void launch_cfg16(const void *a, const void *w, const void *scales, void *c, int
            static_cast<uint32_t *>(workspace));
 }
 
+
+// ---- dequantise once per workgroup --------------------------------------------------------------------------------------
+//
+// gemm_w4a16_kernel16 widens every weight once per wave and M tile; with M in the hundreds or thousands that is
+// several times per weight and the VALU, not the MFMA, sets the pace. Here a workgroup of 8 waves owns 256 rows x 128
+// columns and widens each weight of a 64-row stage ONCE: the packed rows (4 KiB) and the group's scales (256 B) come
+// into an LDS ring by buffer_load ... lds three stages ahead; thread (byte b, 8-row chunk c) reads its 8 bytes (two
+// columns x 8 rows), widens the 16 weights (v_bfe_i32, v_cvt_f32_i32, v_mul, v_cvt_pk) and writes two 16-byte chunks
+// into a double-buffered tile laid out like the activation tile (one 128-byte row of 64 k per output column, chunks
+// swizzled by row), from which every wave reads its B fragments. LDS row r of that tile holds output column
+// (r / 64) * 64 + (r % 16) * 4 + (r / 16) % 4: the 16 lanes of a fragment read 16 consecutive LDS rows (no bank
+// conflicts) and a lane's four MFMA column blocks are four consecutive output columns (8-byte stores).
+//
+// Every LDS access of the kernel is hand-placed asm: the compiler orders any LDS access of its own behind ALL
+// outstanding buffer_load ... lds (it cannot tell which bytes they write), which would serialise the ring.
+
+struct GemmW4LdsCfg {
+    static constexpr int kBM = 256;
+    static constexpr int kBN = 128;
+    static constexpr int kThreads = 512;
+    static constexpr int kAChunks = kBM * 8 / kThreads;
+    static constexpr int kASlotBytes = kBM * 128;
+    static constexpr int kBBufBytes = kBN * 128;
+    static constexpr int kBBase = 3 * kASlotBytes;
+    static constexpr int kRawBase = kBBase + 2 * kBBufBytes;
+    static constexpr int kRawSlotBytes = 64 * 64 + 256;  // 64 rows x 64 bytes, then 128 scales
+    static constexpr int kRingBytes = kRawBase + 3 * kRawSlotBytes;
+    static constexpr int kLdsBytes = kRingBytes + 16;  // + the fix-up's flag; the ring must start at LDS address 0
+    };
+
+template <int OFFSET>
+__device__ __forceinline__ uint32_t lds_read_u8_early(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+__device__ __forceinline__ uint32_t lds_read_b32_early(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+__device__ __forceinline__ void lds_write_b128(uint32_t addr, const uint4v_t &v) {
+    asm volatile("ds_write_b128 %0, %1" : : "v"(addr), "v"(v) : "memory");
+}
+// waits until at most NEWER LDS operations issued after the reads into these registers are outstanding
+template <int NEWER>
+__device__ __forceinline__ void lds_wait_keep_newer(uint32_t (&b)[8], uint32_t &s) {
+    asm volatile("s_waitcnt lgkmcnt(%9)"
+                 : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7]), "+v"(s)
+                 : "n"(NEWER));
+}
+template <int NEWER>
+__device__ __forceinline__ void lds_wait_keep_newer(int4v_t (&f)[4], int4v_t (&g)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(%8)"
+                 : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(g[0]), "+v"(g[1]), "+v"(g[2]), "+v"(g[3])
+                 : "n"(NEWER));
+}
+
+template <int DT>
+__global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
+    const uint16_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ w, const uint16_t *__restrict__ scales,
+    uint16_t *__restrict__ c, int m, int k, int n, int group, int tiles_m, int tiles_n, int xm, int xn, int concurrent,
+    int tail_parts, int tail_stride, float *__restrict__ partials, uint32_t *__restrict__ counters) {
+    using Cfg = GemmW4LdsCfg;
+    using T = W4G<DT>;
+    extern __shared__ uint4 lds[];  // no static LDS in this kernel: every access addresses the ring from 0
+    int &s_last = *reinterpret_cast<int *>(lds + Cfg::kRingBytes / 16);
+
+    GemmWorkItem item;
+    if (!gemm_work_item(tiles_m, tiles_n, xm, xn, concurrent, tail_parts, tail_stride, &item)) return;
+    const int m0 = item.tile_m * Cfg::kBM;
+    const int n0 = item.tile_n * Cfg::kBN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 waves of 64 rows x 64 columns
+    const int kg = lane >> 4, ns = lane & 15;
+
+    float4_t acc[4][4];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[rb][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int row_bytes = n >> 1;
+    const __amdgpu_buffer_rsrc_t rsrc_w =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w), 0, int(int64_t(k) * row_bytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(scales), 0, int(int64_t(k / group) * n * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(a), 0, int((int64_t(m - 1) * lda + k) * 2), 0x00020000);
+
+    constexpr int kOutside = 0x7FFFFFF0;  // rows / columns past the tensor read as zero
+    int a_off[Cfg::kAChunks];
+#pragma unroll
+    for (int j = 0; j < Cfg::kAChunks; ++j) {
+        const int id = j * Cfg::kThreads + tid;
+        const int r = id >> 3;
+        const int row = m0 + r;
+        a_off[j] = row < m ? int((int64_t(row) * lda + ((id & 7) ^ lds_swizzle_key_step1(r)) * 8) * 2) : kOutside;
+    }
+    // packed rows: lanes 0..31 of wave v bring 16 bytes each: row 8v + lane / 4 of the stage, quarter lane % 4 of the
+    // tile's 64 bytes. scales: lanes 0..7 bring one dword (two columns) each. (n % 32 == 0: whole quarters.)
+    const int wq_col = (n0 >> 1) + (lane & 3) * 16;
+    const int wq_off = wq_col < row_bytes ? (lane >> 2) * row_bytes + wq_col : kOutside;
+    const int sq_col = n0 + 2 * (wave * 8 + lane);
+    const int sq_off = sq_col < n ? sq_col * 2 : kOutside;
+
+    const int stages = k / kBK;
+    const int s_begin = (stages * item.part) / item.parts, s_end = (stages * (item.part + 1)) / item.parts;
+
+    // A short matrix leaves most of a 256-row tile empty: a wave skips the activation loads whose 8 rows all lie past
+    // the end (instruction j of wave v brings rows 64 j + 8 v .. + 7) and, if its 64 output rows do, its fragment reads
+    // and MFMAs, so that the stage costs what the widening costs.
+    int a_cnt = 0;
+#pragma unroll
+    for (int j = 0; j < Cfg::kAChunks; ++j) a_cnt += int(m0 + j * 64 + wave * 8 < m);
+    const bool wave_active = m0 + wm * 64 < m;
+
+    auto load_a = [&](int st, int slot, auto all_tag) {
+        // the scalar offset is not part of the buffer's range check: never let it point past the tensor (a prefetch
+        // for a stage past the end re-reads the last stage; its values are not used)
+        const int stc = st < stages ? st : stages - 1;
+#pragma unroll
+        for (int j = 0; j < Cfg::kAChunks; ++j)
+            if (decltype(all_tag)::value || j < a_cnt)
+                buffer_load_to_lds_b128(rsrc_a, lds + slot * Cfg::kBM * 8 + j * Cfg::kThreads + wave * 64, a_off[j], stc * (kBK * 2));
+    };
+    auto wait_older_loads = [&](auto all_tag) {  // all but the loads of the last load_a + load_raw have landed
+        if (decltype(all_tag)::value) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(Cfg::kAChunks + 2));
+            return;
+        }
+        switch (a_cnt) {
+            case 0: __builtin_amdgcn_s_waitcnt(waitcnt_vm(2)); break;
+            case 1: __builtin_amdgcn_s_waitcnt(waitcnt_vm(3)); break;
+            case 2: __builtin_amdgcn_s_waitcnt(waitcnt_vm(4)); break;
+            case 3: __builtin_amdgcn_s_waitcnt(waitcnt_vm(5)); break;
+            default: __builtin_amdgcn_s_waitcnt(waitcnt_vm(6)); break;
+        }
+    };
+    auto load_raw = [&](int st, int slot) {
+        const int stc = st < stages ? st : stages - 1;
+        char *dst = reinterpret_cast<char *>(lds) + Cfg::kRawBase + slot * Cfg::kRawSlotBytes;
+        if (lane < 32)
+            buffer_load_to_lds_b128(rsrc_w, reinterpret_cast<uint4 *>(dst + wave * 512), wq_off, (stc * kBK + wave * 8) * row_bytes);
+        if (lane < 8)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_s, (__attribute__((address_space(3))) void *)(dst + 4096 + wave * 32),
+                                                     4, sq_off, ((stc * kBK) / group) * n * 2, 0, 0);
+    };
+
+    // Dequantisation: thread (lane, wave) widens bytes `lane` (columns 2 lane, 2 lane + 1) of rows 8 wave .. 8 wave + 7.
+    const uint32_t raw_rd = uint32_t(Cfg::kRawBase + wave * 512 + lane);
+    const uint32_t sc_rd = uint32_t(Cfg::kRawBase + 4096 + lane * 4);
+    uint32_t bw_addr[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const int sig = (lane >> 5) * 64 + (2 * (lane & 1) + e) * 16 + ((lane & 31) >> 1);
+        bw_addr[e] = uint32_t(Cfg::kBBase + (sig * 8 + (wave ^ lds_swizzle_key_step1(sig))) * 16);
+    }
+    uint32_t bytes[8], sc2;
+    auto read_raw = [&](int slot) {
+        const uint32_t base = raw_rd + slot * Cfg::kRawSlotBytes;
+        bytes[0] = lds_read_u8_early<0 * 64>(base);
+        bytes[1] = lds_read_u8_early<1 * 64>(base);
+        bytes[2] = lds_read_u8_early<2 * 64>(base);
+        bytes[3] = lds_read_u8_early<3 * 64>(base);
+        bytes[4] = lds_read_u8_early<4 * 64>(base);
+        bytes[5] = lds_read_u8_early<5 * 64>(base);
+        bytes[6] = lds_read_u8_early<6 * 64>(base);
+        bytes[7] = lds_read_u8_early<7 * 64>(base);
+        sc2 = lds_read_b32_early(sc_rd + slot * Cfg::kRawSlotBytes);
+    };
+    uint4v_t chunk[2];
+    auto dequant = [&]() {  // q * scale is exact in fp32: one rounding, to the 16-bit type
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float sv = T::to_f32(uint16_t(sc2 >> (16 * e)));
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int q0 = int(bytes[2 * p] << (28 - 4 * e)) >> 28, q1 = int(bytes[2 * p + 1] << (28 - 4 * e)) >> 28;
+                chunk[e][p] = T::pack2(float(q0) * sv, float(q1) * sv);
+            }
+        }
+    };
+
+    // LDS byte addresses of this lane's A fragment (row block 0, ring slot 0) and B fragment (column block 0, buffer 0)
+    uint32_t af_addr[2], bf_addr[2];
+    {
+        const int ra = wm * 64 + ns, rb_ = wn * 64 + ns;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            af_addr[q] = uint32_t((ra * 8 + ((q * 4 + kg) ^ lds_swizzle_key_step1(ra))) * 16);
+            bf_addr[q] = uint32_t(Cfg::kBBase + (rb_ * 8 + ((q * 4 + kg) ^ lds_swizzle_key_step1(rb_))) * 16);
+        }
+    }
+    int4v_t af[2][4], bf[2][4];
+    auto read_frags = [&](int4v_t (&dst)[4], uint32_t addr) {
+        dst[0] = lds_read_b128_early<0 * 2048>(addr);
+        dst[1] = lds_read_b128_early<1 * 2048>(addr);
+        dst[2] = lds_read_b128_early<2 * 2048>(addr);
+        dst[3] = lds_read_b128_early<3 * 2048>(addr);
+    };
+    auto mfmas = [&](int4v_t (&fa)[4], int4v_t (&fb)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb)
+                acc[rb][t] = T::mfma(__builtin_bit_cast(uint4, fa[rb]), __builtin_bit_cast(uint4, fb[t]), acc[rb][t]);
+    };
+
+    // Schedule. One barrier per stage, in the middle: M(s). Stage s runs as
+    //   H1(s): MFMAs of k-step 0 with the widening of stage s + 1 (bytes read during H2(s-1)) in their shadow, then
+    //          the two tile writes into the other buffer
+    //   M(s):  own LDS traffic done, own loads of H2(s-2) landed, barrier
+    //   H2(s): reads of the bytes of stage s + 2 and of the k-step 0 fragments of stage s + 1; MFMAs of k-step 1 with
+    //          the loads of activations s + 3 and packed rows s + 4 between them; then the reads of the k-step 1
+    //          fragments of stage s + 1 into the registers just consumed
+    // so every LDS read has half a stage to land and the only LDS traffic between the last MFMA of H1 and the barrier
+    // is the two writes. Ring slot of stage x is (x - s_begin) % 3 for activations and packed rows, tile buffer
+    // (x - s_begin) % 2.
+    auto mfmas_half = [&](int4v_t (&fa)[4], int4v_t (&fb)[4], int t0) {
+#pragma unroll
+        for (int t = t0; t < t0 + 2; ++t)
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb)
+                acc[rb][t] = T::mfma(__builtin_bit_cast(uint4, fa[rb]), __builtin_bit_cast(uint4, fb[t]), acc[rb][t]);
+    };
+    load_raw(s_begin, 0);
+    load_a(s_begin, 0, std::false_type());
+    load_raw(s_begin + 1, 1);
+    load_a(s_begin + 1, 1, std::false_type());
+    load_raw(s_begin + 2, 2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __builtin_amdgcn_s_barrier();
+    read_raw(0);
+    lds_wait_keep_newer<0>(bytes, sc2);
+    dequant();
+    lds_write_b128(bw_addr[0], chunk[0]);
+    lds_write_b128(bw_addr[1], chunk[1]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    load_a(s_begin + 2, 2, std::false_type());
+    load_raw(s_begin + 3, 0);
+    read_raw(1);
+    auto active_loop = [&](auto all_tag) {
+        read_frags(af[0], af_addr[0]);
+        read_frags(bf[0], bf_addr[0]);
+        read_frags(af[1], af_addr[1]);
+        read_frags(bf[1], bf_addr[1]);
+        for (int s = s_begin, slot = 0, buf = 0; s < s_end; ++s) {
+            const int slot1 = slot == 2 ? 0 : slot + 1, slot2 = slot >= 1 ? slot - 1 : 2;
+            const uint32_t a_next = uint32_t(slot1 * Cfg::kASlotBytes), b_other = uint32_t((buf ^ 1) * Cfg::kBBufBytes);
+            // H1
+            lds_wait_keep_newer<8>(bytes, sc2);
+            lds_wait_keep_newer<8>(af[0], bf[0]);
+            dequant();
+            mfmas(af[0], bf[0]);
+            // the two waves of a SIMD run in step: widening must sit in the shadow of this wave's own MFMAs, or the
+            // MFMA pipe idles while both widen
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // four VALU
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            lds_write_b128(bw_addr[0] + b_other, chunk[0]);
+            lds_write_b128(bw_addr[1] + b_other, chunk[1]);
+            lds_wait_keep_newer<0>(af[1], bf[1]);
+            wait_older_loads(all_tag);
+            __builtin_amdgcn_s_barrier();
+            // H2
+            read_raw(slot2);
+            read_frags(af[0], af_addr[0] + a_next);
+            read_frags(bf[0], bf_addr[0] + b_other);
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas_half(af[1], bf[1], 0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_a(s + 3, slot, all_tag);
+            load_raw(s + 4, slot1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas_half(af[1], bf[1], 2);
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(af[1], af_addr[1] + a_next);
+            read_frags(bf[1], bf_addr[1] + b_other);
+            slot = slot1;
+            buf ^= 1;
+        }
+        // drain: the reads issued for the stage past the end are not used, but their registers must not be reused
+        // before they have landed
+        lds_wait_keep_newer<0>(af[0], bf[0]);
+        lds_wait_keep_newer<0>(af[1], bf[1]);
+    };
+    if (a_cnt == Cfg::kAChunks) {  // then the wave is active too
+        active_loop(std::true_type());
+    } else if (wave_active) {
+        active_loop(std::false_type());
+    } else {
+        // same loads, widening, writes and barriers; no fragments, no MFMAs
+        for (int s = s_begin, slot = 0, buf = 0; s < s_end; ++s) {
+            const int slot1 = slot == 2 ? 0 : slot + 1, slot2 = slot >= 1 ? slot - 1 : 2;
+            const uint32_t b_other = uint32_t((buf ^ 1) * Cfg::kBBufBytes);
+            lds_wait_keep_newer<0>(bytes, sc2);
+            dequant();
+            lds_write_b128(bw_addr[0] + b_other, chunk[0]);
+            lds_write_b128(bw_addr[1] + b_other, chunk[1]);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            wait_older_loads(std::false_type());
+            __builtin_amdgcn_s_barrier();
+            read_raw(slot2);
+            load_a(s + 3, slot, std::false_type());
+            load_raw(s + 4, slot1);
+            slot = slot1;
+            buf ^= 1;
+        }
+    }
+    lds_wait_keep_newer<0>(bytes, sc2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // LDS must not be released with loads in flight
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (item.parts > 1) {
+        uint32_t rows_valid = 0;  // row blocks of this wave that reach into the matrix
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) rows_valid |= uint32_t(m0 + wm * 64 + rb * 16 < m) << rb;
+        if (!gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last, rows_valid)) return;
+    }
+
+    const int col = n0 + wn * 64 + ns * 4;  // first of this lane's 4 columns
+    if (col >= n) return;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int row = m0 + wm * 64 + rb * 16 + kg * 4 + v;
+            if (row < m) {
+                uint2 o;
+                o.x = uint32_t(T::from_f32(acc[rb][0][v])) | (uint32_t(T::from_f32(acc[rb][1][v])) << 16);
+                o.y = uint32_t(T::from_f32(acc[rb][2][v])) | (uint32_t(T::from_f32(acc[rb][3][v])) << 16);
+                *reinterpret_cast<uint2 *>(c + int64_t(row) * n + col) = o;
+            }
+        }
+}
+
+template <int DT>
+void launch_lds(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                int group, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    using Cfg = GemmW4LdsCfg;
+    const int tiles_m = int(cdiv(m, Cfg::kBM)), tiles_n = int(cdiv(n, Cfg::kBN));
+    constexpr int kConcurrent = 32;
+    const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
+    GemmTail tail = make_gemm_tail(tiling, kConcurrent, kConcurrent, 4);
+    while (tail.parts > 1 &&
+           (k / kBK < 8 * tail.parts ||
+            workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
+        --tail.parts;
+    const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
+    QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
+    static bool attr_set = false;
+    if (!attr_set) {
+        QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a16_lds_kernel<DT>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
+        attr_set = true;
+    }
+    launch(gemm_w4a16_lds_kernel<DT>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
+           static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
+           static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,
+           tail.parts, tail.max_tiles, reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes),
+           static_cast<uint32_t *>(workspace));
+}
+
 }  // namespace
 
 bool gemm_w4a16_supported(const void *a, const void *w, const void *scales, const void *c, int64_t k, int64_t n,
@@ -477,6 +855,14 @@ void gemm_w4a16_launch(const void *a, const void *w, const void *scales, void *c
                        int64_t lda, int group, int dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     const bool fast = (k % kBK == 0) && (group % kBK == 0) && k * (n / 2) < (int64_t(1) << 31) - (1 << 20) &&
                       (m * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20) && (k / group) * n * 2 < (int64_t(1) << 31);
+    // Measured on K = 4096, N = 11008, M = 33 .. 4096: the kernel that widens once per workgroup (256-row tiles) is
+    // ahead except where its tall tiles leave a second or third tile row mostly empty (3 or 5 tile rows of 128).
+    const int64_t rows128 = cdiv(m, 128);
+    if (fast && n % 32 == 0 && rows128 != 3 && rows128 != 5) {
+        if (dtype == HIDET_QMM_F16) launch_lds<HIDET_QMM_F16>(a, w, scales, c, m, k, n, lda, group, workspace, workspace_bytes, stream);
+        else launch_lds<HIDET_QMM_BF16>(a, w, scales, c, m, k, n, lda, group, workspace, workspace_bytes, stream);
+        return;
+    }
     if (fast) {
         // workgroup tile 128 x 256: 4 waves of 64 x 128, two workgroups per CU
         if (dtype == HIDET_QMM_F16) launch_cfg16<HIDET_QMM_F16, 4, 2, 2, 2>(a, w, scales, c, m, k, n, lda, group, workspace, workspace_bytes, stream);

@@ -216,7 +216,12 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
 
     // a tile computed in K ranges is finished by the part that arrives last (gemm_k_split_fixup)
-    if (parts > 1 && !gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last)) return;
+    if (parts > 1) {
+        uint32_t rows_valid = 0;  // row blocks of this wave that reach into the matrix
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) rows_valid |= uint32_t(m0 + (wm * RB + rb) * 16 < m) << rb;
+        if (!gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last, rows_valid)) return;
+    }
 
     // acc[rb][t][v] = c[m0 + (wm*RB + rb)*16 + 4*kg + v][col + t]
     if (!col_ok) return;

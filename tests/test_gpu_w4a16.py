@@ -58,7 +58,11 @@ def test_skinny_parity(m, k, n, g, dtype):
 
 
 @pytest.mark.parametrize('m,k,n,g', [(128, 256, 256, 128), (65, 128, 264, 32), (512, 4096, 1024, 128), (300, 512, 520, 64),
-                                     (33, 4096, 512, 128), (40, 512, 264, 64), (24, 512, 256, 128)])
+                                     (33, 4096, 512, 128), (40, 512, 264, 64), (24, 512, 256, 128),
+                                     # 256-row tiles widened once per workgroup: a short last tile, K split with mostly
+                                     # empty tiles, a ragged last column tile, waves without rows
+                                     (129, 4096, 512, 128), (500, 512, 544, 64), (1000, 256, 1056, 128),
+                                     (40, 4096, 544, 128), (70, 1024, 2080, 64)])
 @pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
 def test_gemm_parity(m, k, n, g, dtype):
     announce('w4a16 gemm', m, k, n, g, dtype)
@@ -74,7 +78,7 @@ def test_gemm_parity(m, k, n, g, dtype):
 def test_exact_on_small_integers():
     announce('w4a16 exact')
     rng = np.random.default_rng(21)
-    for (m, k, n) in ((4, 256, 256), (128, 256, 128)):
+    for (m, k, n) in ((4, 256, 256), (128, 256, 128), (200, 4096, 256), (48, 4096, 1024)):  # the last two split K
         a = rng.integers(-3, 4, (m, k)).astype(np.float32)
         q = rng.integers(-8, 8, (k, n)).astype(np.int8)  # -8 is representable and must decode correctly
         scales = (2.0 ** rng.integers(-3, 1, (k // 128, n))).astype(np.float32)
@@ -83,6 +87,15 @@ def test_exact_on_small_integers():
             want += (a[:, g * 128:(g + 1) * 128].astype(np.int64) @ q[g * 128:(g + 1) * 128].astype(np.int64)) * scales[g]
         got = host(quant.symmetric_quant_matmul_w4a16(dev(a, torch.bfloat16), dev(O.pack_int4(q)), dev(scales, torch.bfloat16), 128))
         assert np.array_equal(got, O.to_bf16(want.astype(np.float32))), (m, k, n)
+
+
+def test_k_split_is_deterministic():
+    m, k, n, g = 129, 4096, 512, 128
+    announce('w4a16 k split twice', m, k, n)
+    _, _, _, ta, tp, ts = _case(3, m, k, n, g, 'bfloat16')
+    first = host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g))
+    for _ in range(3):
+        assert np.array_equal(host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g)), first)
 
 
 def test_full_size_prefill_rows_sample():
