@@ -19,7 +19,8 @@
 // ahead into the registers they were just dequantised from.  The activation tile goes global -> LDS
 // directly (buffer_load ... lds, no registers) into a three-slot ring of 16-byte chunks XOR-swizzled by
 // row (the swizzle is applied on the global side), two stages ahead; one barrier per 64 k.  The per-column
-// scale is applied to the fp32 accumulators in the epilogue.
+// scale is applied to the fp32 accumulators in the epilogue.  Matrices of at most 96 rows run the same tile with the
+// row blocks that cannot hold a row left out at compile time (template parameter RBA).
 #include "common.h"
 #include "gemm_tiling.h"
 
@@ -38,7 +39,9 @@ struct GemmW8Cfg16 {
     static constexpr int kLdsBytes = kRingBytes + 16;  // + the fix-up's flag; the ring must start at LDS address 0
 };
 
-template <int RB, int WM, int WN, int MIN_BLOCKS>
+// RBA <= RB: row blocks (of 16 rows) per wave that can hold rows of the matrix. A short matrix (M <= 16 RBA) runs the same
+// tile with the activation loads, fragment reads and MFMAs of the other row blocks left out.
+template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA>
 __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(const _Float16 *__restrict__ a, int64_t lda,
                                                                                  const int8_t *__restrict__ w,
                                                                                  const _Float16 *__restrict__ scale,
@@ -101,9 +104,12 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     };
     BFrag bq[2][4];
 
+    // instruction j brings tile rows j * kThreads / 8 ..: only those below 16 RBA are needed
+    static_assert(WM == 1 && (RBA * 16 * 8) % Cfg::kThreads == 0, "whole load instructions per active row range");
+    constexpr int kAChunksActive = RBA * 16 * 8 / Cfg::kThreads;
     auto load_a = [&](int st, int slot) {
 #pragma unroll
-        for (int j = 0; j < Cfg::kAChunks; ++j)
+        for (int j = 0; j < kAChunksActive; ++j)
             buffer_load_to_lds_b128(rsrc_a, lds + slot * Cfg::kBM * 8 + j * Cfg::kThreads + wave * 64, a_off[j], st * (kBK * 2));
     };
     auto load_w = [&](int st, int q, uint32_t (&dst)[8]) {
@@ -137,10 +143,11 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         const uint32_t slot_off = uint32_t(slot * Cfg::kBM * 128);
         const uint32_t addr0 = af_addr[0] + slot_off, addr1 = af_addr[1] + slot_off;
         // A fragments are read from LDS three fragments (12 MFMAs) ahead of their use, through a ring of four
+        // (fragment index = k-step * RBA + row block, over the active row blocks only)
         int4v_t af[4];
         auto issue = [&](auto idx_tag) {
             constexpr int IDX = decltype(idx_tag)::value;
-            if constexpr (IDX < 2 * RB) af[IDX & 3] = lds_read_b128_early<(IDX % RB) * 2048>(IDX / RB ? addr1 : addr0);
+            if constexpr (IDX < 2 * RBA) af[IDX & 3] = lds_read_b128_early<(IDX % RBA) * 2048>(IDX / RBA ? addr1 : addr0);
         };
         issue(std::integral_constant<int, 0>());
         issue(std::integral_constant<int, 1>());
@@ -150,7 +157,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         auto block = [&](auto idx_tag) {
             constexpr int IDX = decltype(idx_tag)::value;
             constexpr int Q = IDX / RB, RBI = IDX % RB;
-            issue(std::integral_constant<int, IDX + 3>());
+            constexpr int AI = Q * RBA + RBI;  // fragment index, if the row block is active
+            if constexpr (RBI < RBA) issue(std::integral_constant<int, AI + 3>());
             {
                 constexpr int P = RBI / 2;  // row pair of the next k-step's raw block
 #pragma unroll
@@ -171,12 +179,14 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
                     w_raw[Q ^ 1][2 * P + 1] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[2 * P + 1], soff, 0);
                 }
             }
-            constexpr int NEWER = (2 * RB - 1 - IDX) < 3 ? (2 * RB - 1 - IDX) : 3;
-            lds_wait_keep_newer<NEWER>(af[IDX & 3]);
-            const half8_t afrag = __builtin_bit_cast(half8_t, af[IDX & 3]);
+            if constexpr (RBI < RBA) {
+                constexpr int NEWER = (2 * RBA - 1 - AI) < 3 ? (2 * RBA - 1 - AI) : 3;
+                lds_wait_keep_newer<NEWER>(af[AI & 3]);
+                const half8_t afrag = __builtin_bit_cast(half8_t, af[AI & 3]);
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                acc[RBI][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bq[Q][t].h8, acc[RBI][t], 0, 0, 0);
+                for (int t = 0; t < 4; ++t)
+                    acc[RBI][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bq[Q][t].h8, acc[RBI][t], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         };
         auto kstep = [&](auto q_tag) {
@@ -194,8 +204,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         kstep(std::integral_constant<int, 0>());
         kstep(std::integral_constant<int, 1>());
         // the loads of stage s + 1 (issued one stage ago) must have landed in LDS before anyone reads them; the
-        // loads issued during this stage (kAChunks + 16 of them) may stay in flight
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(Cfg::kAChunks + 16));
+        // loads issued during this stage (kAChunksActive + 16 of them) may stay in flight
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(kAChunksActive + 16));
         __syncthreads();
     };
 
@@ -219,8 +229,11 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     if (parts > 1) {
         uint32_t rows_valid = 0;  // row blocks of this wave that reach into the matrix
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) rows_valid |= uint32_t(m0 + (wm * RB + rb) * 16 < m) << rb;
-        if (!gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last, rows_valid)) return;
+        for (int rb = 0; rb < RBA; ++rb) rows_valid |= uint32_t(m0 + (wm * RB + rb) * 16 < m) << rb;
+        // only the active row blocks take part (every workgroup of a launch has the same RBA)
+        if (!gemm_k_split_fixup<Cfg::kThreads>(reinterpret_cast<float4_t(&)[RBA][4]>(acc), item, partials, counters, &s_last,
+                                               rows_valid))
+            return;
     }
 
     // acc[rb][t][v] = c[m0 + (wm*RB + rb)*16 + 4*kg + v][col + t]
@@ -229,7 +242,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
 #pragma unroll
     for (int t = 0; t < 4; ++t) sc[t] = float(scale[col + t]);
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+    for (int rb = 0; rb < RBA; ++rb)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int row = m0 + (wm * RB + rb) * 16 + kg * 4 + v;
@@ -242,7 +255,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         }
 }
 
-template <int RB, int WM, int WN, int MIN_BLOCKS>
+template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA>
 void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
                   void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     using Cfg = GemmW8Cfg16<RB, WM, WN>;
@@ -251,7 +264,8 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
     // Tail split: at most 4 K ranges of at least 8 stages each, and only with workspace for the partial tiles
     // (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
-    GemmTail tail = make_gemm_tail(tiling, kConcurrent, 32, 4);
+    // (light workgroups - at most 4 active row blocks - are worth up to 8 ranges: measured)
+    GemmTail tail = make_gemm_tail(tiling, kConcurrent, 32, RBA <= 4 ? 8 : 4);
     while (tail.parts > 1 &&
            (k / kBK < 8 * tail.parts ||
             workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
@@ -262,12 +276,12 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     if (Cfg::kLdsBytes > 65536) {
         static bool attr_set = false;
         if (!attr_set) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS>),
+            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
             attr_set = true;
         }
     }
-    launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
+    launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale),
            static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent, tail.parts, tail.max_tiles,
            reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
@@ -284,7 +298,11 @@ bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m
 
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
-    launch_cfg16<8, 1, 4, 2>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);  // waves 128 x 64, workgroup tile 128 x 256
+    // waves 128 x 64, workgroup tile 128 x 256; a matrix of at most 32 / 64 / 96 rows leaves the empty row blocks out
+    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
+    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
+    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
+    else launch_cfg16<8, 1, 4, 2, 8>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
 }
 
 }  // namespace qmm
