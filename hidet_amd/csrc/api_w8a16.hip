@@ -23,10 +23,13 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
     QMM_CHECK(a && w && scale && c, "null tensor pointer");
     QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    // Up to 16 rows one pass of the bandwidth-bound kernel is fastest (21 us at K=4096, N=11008). Beyond that every 16
-    // rows cost another pass over the weights (36 us at M=17, 79 us at M=64) while the MFMA GEMM with its K split takes
-    // 28 us for any M up to 128.
-    if (m > 16 && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
+    // Up to 16 rows one pass of the bandwidth-bound kernel serves; beyond that every 16 rows would cost another pass
+    // over the weights, and the MFMA GEMM with its K split and its empty row blocks left out takes over (K=4096, N=11008,
+    // weights from HBM: 17 us at M=17..32, 20 us at M=64, 29 us at M=128). From 9 rows on the GEMM is already ahead when
+    // the output is wide enough for its 256-column tiles to fill the chip (N=11008: 16.0 against 18.4 us; N=4096: 13.6
+    // against 13.4 us), unless the caller asked for a specific K split of the bandwidth-bound kernel.
+    const bool wide = cdiv(n, 256) >= 32;
+    if ((m > 16 || (m > 8 && wide && parallel_k_parts == 0)) && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
         gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
         skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);

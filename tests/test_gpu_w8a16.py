@@ -30,7 +30,8 @@ def _int_case(seed, m, k, n):
 
 
 @pytest.mark.parametrize('m,k,n', [(1, 256, 256), (1, 4096, 512), (3, 1024, 768), (16, 512, 256), (7, 96, 48),
-                                   (1, 40, 16), (2, 8, 16), (1, 4096, 272), (16, 4096, 4096)])
+                                   (1, 40, 16), (2, 8, 16), (1, 4096, 272), (16, 4096, 4096),
+                                   (9, 4096, 8192), (16, 1024, 11008), (12, 512, 8200)])  # wide outputs: 9+ rows take the MFMA GEMM
 def test_exact_on_small_integers(m, k, n):
     # integer activations and codes with power-of-two scales: every product and partial sum is exact in
     # fp32, so any dropped row, wrong byte or lost K slice shows as a whole-number difference
@@ -59,7 +60,7 @@ def test_reference_recipe(x_shape, w_shape):
 
 @pytest.mark.parametrize('m,k,n,seed', [(16, 4096, 4096, 0), (1, 4096, 11008, 0), (1, 4096, 11008, 1),
                                         (1, 4096, 11008, 2), (1, 4096, 11008, 3), (1, 11008, 4096, 0),
-                                        (1, 11008, 4096, 3), (5, 1000, 528, 0), (33, 512, 256, 0)])
+                                        (1, 11008, 4096, 3), (5, 1000, 528, 0), (33, 512, 256, 0), (13, 4096, 11008, 0)])
 def test_parity_with_oracle(m, k, n, seed):
     announce('w8a16 parity', m, k, n, seed)
     a, q, s = _case(seed, m, k, n)
