@@ -227,7 +227,7 @@ def main():
     c8 = torch.empty((MF, NF), dtype=torch.bfloat16, device=device)
 
     def launch_fp8(i):
-        ffi.call('hidet_matmul_f8', a8, b8s[i][0], c8, MF, NF, KF, KF, KF, 2, sa, b8s[i][1], sptr)
+        ffi.call('hidet_matmul_f8', a8, b8s[i][0], c8, MF, NF, KF, KF, KF, 2, sa, b8s[i][1], work, work.numel(), sptr)
 
     with torch.cuda.stream(stream):
         for i in range(3):
@@ -310,7 +310,7 @@ def main():
     a1 = a8[:1].contiguous()
     c1 = torch.empty((1, NF), dtype=torch.bfloat16, device=device)
     bring = [bq for bq, _ in b8s] + [torch.randint(0, 0x7F, (NF, KF), device=device, dtype=torch.uint8) for _ in range(5)]  # 8 x 64 MiB
-    us = time_kernel(lambda r: ffi.call('hidet_matmul_f8', a1, bring[r % 8], c1, 1, NF, KF, KF, KF, 2, sa, b8s[0][1], sptr), 32, 8)
+    us = time_kernel(lambda r: ffi.call('hidet_matmul_f8', a1, bring[r % 8], c1, 1, NF, KF, KF, KF, 2, sa, b8s[0][1], work, work.numel(), sptr), 32, 8)
     del bring
     others['fp8_gemv_m1_k8192_n8192'] = hbm_entry(us, NF * KF + KF + 2 * NF + 8)
 
@@ -330,7 +330,7 @@ def main():
         a8z, b8z = torch.zeros_like(a8.view(torch.uint8)), torch.zeros_like(b8s[0][0].view(torch.uint8))
         w8_zero = timed(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', az, wz, ss[0], cp, MP, K, N, K, 0, work,
                                            work.numel(), sptr))
-        f8_zero = timed(lambda r: ffi.call('hidet_matmul_f8', a8z, b8z, c8, MF, NF, KF, KF, KF, 2, sa, b8s[0][1], sptr))
+        f8_zero = timed(lambda r: ffi.call('hidet_matmul_f8', a8z, b8z, c8, MF, NF, KF, KF, KF, 2, sa, b8s[0][1], work, work.numel(), sptr))
         print(json.dumps({'data_dependence': {
             'w8a16_gemm_us': {'benchmark_operands': round(float(pd.mean()), 2), 'zero_operands': round(w8_zero, 2)},
             'fp8_gemm_us': {'benchmark_operands': round(float(fd.mean()), 2), 'zero_operands': round(f8_zero, 2)}}}))

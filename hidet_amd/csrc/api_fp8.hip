@@ -6,12 +6,20 @@ bool skinny_fp8_supported(const void *b, int64_t k, int64_t ldb);
 void skinny_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
                        int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
 void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
-                     int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
+                     int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
+                     hipStream_t stream);
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                            int64_t n, int64_t k, int out_dtype, hipStream_t stream);
+                            int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 }  // namespace qmm
 
 using namespace qmm;
+
+// The workspace is optional here (NULL: tiles are never computed in K ranges); when given it starts with the 64 KiB of
+// arrival counters, which are zero between calls.
+static void check_workspace(const void *workspace, int64_t workspace_bytes) {
+    QMM_CHECK(workspace_bytes >= 0, "negative workspace size");
+    QMM_CHECK(workspace == nullptr || aligned(workspace, 16), "the workspace must be 16-byte aligned");
+}
 
 static void check_out_dtype(int out_dtype) {
     QMM_CHECK(out_dtype == HIDET_QMM_F32 || out_dtype == HIDET_QMM_F16 || out_dtype == HIDET_QMM_BF16 || out_dtype == HIDET_QMM_E4M3,
@@ -19,7 +27,8 @@ static void check_out_dtype(int out_dtype) {
 }
 
 HIDET_API void hidet_matmul_f8(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda,
-                               int64_t ldb, int out_dtype, const void *scale_a, const void *scale_b, void *stream_) {
+                               int64_t ldb, int out_dtype, const void *scale_a, const void *scale_b, void *workspace,
+                               int64_t workspace_bytes, void *stream_) {
     QMM_ENTRY_BEGIN
     check_out_dtype(out_dtype);
     QMM_CHECK(m >= 0 && n >= 0 && k >= 0, "negative extent: m=" << m << " n=" << n << " k=" << k);
@@ -27,16 +36,18 @@ HIDET_API void hidet_matmul_f8(const void *a, const void *b, void *c, int64_t m,
     QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
     if (m == 0 || n == 0) return;
     QMM_CHECK(c && (k == 0 || (a && b)), "null tensor pointer");
+    check_workspace(workspace, workspace_bytes);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (m <= 16 && skinny_fp8_supported(b, k, ldb))
         skinny_fp8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
     else
-        gemm_fp8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
+        gemm_fp8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, workspace, workspace_bytes, stream);
     QMM_ENTRY_END
 }
 
 HIDET_API void hidet_matmul_f8_scaled(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c,
-                                      int64_t m, int64_t n, int64_t k, int out_dtype, void *stream_) {
+                                      int64_t m, int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes,
+                                      void *stream_) {
     QMM_ENTRY_BEGIN
     check_out_dtype(out_dtype);
     QMM_CHECK(m >= 0 && n >= 0 && k >= 0, "negative extent: m=" << m << " n=" << n << " k=" << k);
@@ -47,6 +58,7 @@ HIDET_API void hidet_matmul_f8_scaled(const void *a, const void *b, const void *
     QMM_CHECK(a && b && c && scale_a && scale_b, "null tensor pointer");
     QMM_CHECK(k > 0, "K must be positive");
     QMM_CHECK(aligned(a, 16) && aligned(b, 16) && aligned(c, 16), "tensors must be 16-byte aligned");
-    gemm_fp8_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, static_cast<hipStream_t>(stream_));
+    check_workspace(workspace, workspace_bytes);
+    gemm_fp8_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

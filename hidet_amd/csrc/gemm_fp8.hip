@@ -403,10 +403,12 @@ void dispatch_out(int out_dtype, F &&f) {
 }  // namespace
 
 void gemm_fp8_kernel8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
-                             int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
+                             int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
+                             hipStream_t stream);
 
 void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
-                     int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
+                     int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
+                     hipStream_t stream) {
     const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
     const float *sa = static_cast<const float *>(scale_a), *sb = static_cast<const float *>(scale_b);
     const bool tiled = (k % 16 == 0) && (lda % 16 == 0) && (ldb % 16 == 0) && (n % 4 == 0) && aligned(a, 16) &&
@@ -436,7 +438,7 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
             const int64_t t256 = int64_t(tiles_m) * tiles_n, t128 = int64_t(tiles_m) * cdiv(n, 128);
             const double cost256 = double(cdiv(t256, 256)), cost128 = double(cdiv(t128, 256)) * 0.5 * 1.15;
             if (cost128 < cost256) {
-                gemm_fp8_kernel8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
+                gemm_fp8_kernel8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, workspace, workspace_bytes, stream);
                 return;
             }
             static bool fast_attr_set = false;

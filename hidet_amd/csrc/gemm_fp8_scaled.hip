@@ -154,7 +154,8 @@ constexpr int kM8 = 256, kN8 = 128;           // workgroup tile
 constexpr int kThreads8 = 512;
 constexpr int kSlotChunks8 = (kM8 + kN8) * 8;  // 16-byte chunks of one k block: A rows then B rows
 constexpr int kLoads8 = kSlotChunks8 / kThreads8;  // 6 direct-to-LDS loads per thread and k block
-constexpr int kLdsBytes8 = 3 * kSlotChunks8 * 16;  // 144 KiB
+constexpr int kRingBytes8 = 3 * kSlotChunks8 * 16;  // 144 KiB
+constexpr int kLdsBytes8 = kRingBytes8 + 16;       // + the K-split fix-up's flag; the ring must start at LDS address 0
 
 template <int OUT>
 __device__ __forceinline__ void store4_scaled(void *c, int64_t o, float4_t v) {
@@ -190,12 +191,18 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
                                                                  const uint8_t *__restrict__ b, int64_t ldb,
                                                                  const float *__restrict__ scale_a,
                                                                  const float *__restrict__ scale_b, void *__restrict__ c,
-                                                                 int m, int n, int k, int tiles_m, int tiles_n, int xm, int xn) {
+                                                                 int m, int n, int k, int tiles_m, int tiles_n, int xm, int xn,
+                                                                 int tail_parts, int tail_stride, float *__restrict__ partials,
+                                                                 uint32_t *__restrict__ counters) {
     extern __shared__ uint4 lds[];  // [3][kSlotChunks8]; no static LDS: fragment reads address the ring from 0
-    int tile_m, tile_n;
-    if (!gemm_tile_of_block(tiles_m, tiles_n, xm, xn, &tile_m, &tile_n)) return;
+    int &s_last = *reinterpret_cast<int *>(lds + kRingBytes8 / 16);
+    GemmWorkItem item;
+    if (!gemm_work_item(tiles_m, tiles_n, xm, xn, 32, tail_parts, tail_stride, &item)) return;
+    const int tile_m = item.tile_m, tile_n = item.tile_n;
     const int m0 = tile_m * kM8, n0 = tile_n * kN8;
     const int kblocks = k / 128;
+    // this workgroup's K range (the whole of K unless the launch splits tail tiles)
+    const int kb_begin = (kblocks * item.part) / item.parts, kb_end = (kblocks * (item.part + 1)) / item.parts;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -229,10 +236,35 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
         if (j < 4) voff[j] = m0 + r < m ? int(int64_t(m0 + r) * lda) + chunk * 16 : kOutside;
         else voff[j] = n0 + r - kM8 < n ? int(int64_t(n0 + r - kM8) * ldb) + chunk * 16 : kOutside;
     }
-    auto load_tiles = [&](int kb, int slot) {  // k blocks at and past the end stay inside the buffer or read zero
+    // A short matrix leaves most of the 256 tile rows empty: load instructions whose 64 rows all lie past M are left
+    // out (a_cnt of the 4 stay; the same for every wave), and a wave whose 64 output rows do skips its fragment reads
+    // and MFMAs.
+    int a_cnt = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a_cnt += int(m0 + j * 64 < m);
+    const bool wave_active = m0 + wm * 64 < m;
+    // (all_tag: the tile is full - no conditions in the loop)
+    auto load_tiles = [&](int kb, int slot, auto all_tag) {
+        // the scalar offset is not part of the buffer's range check: a prefetch past the end of K re-reads the last block
+        const int kbc = kb < kblocks ? kb : kblocks - 1;
         uint4 *dst = lds + slot * kSlotChunks8 + wave * 64;
 #pragma unroll
-        for (int j = 0; j < kLoads8; ++j) buffer_load_to_lds_b128(j < 4 ? rsrc_a : rsrc_b, dst + j * kThreads8, voff[j], kb * 128);
+        for (int j = 0; j < kLoads8; ++j)
+            if (decltype(all_tag)::value || j >= 4 || j < a_cnt)
+                buffer_load_to_lds_b128(j < 4 ? rsrc_a : rsrc_b, dst + j * kThreads8, voff[j], kbc * 128);
+    };
+    auto wait_older_tiles = [&](auto all_tag) {  // everything but the loads of the last load_scales + load_tiles has landed
+        constexpr int kScaleLoads = SCALED ? 5 : 0;
+        if (decltype(all_tag)::value) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(kScaleLoads + kLoads8));
+            return;
+        }
+        switch (a_cnt) {
+            case 1: __builtin_amdgcn_s_waitcnt(waitcnt_vm(kScaleLoads + 3)); break;
+            case 2: __builtin_amdgcn_s_waitcnt(waitcnt_vm(kScaleLoads + 4)); break;
+            case 3: __builtin_amdgcn_s_waitcnt(waitcnt_vm(kScaleLoads + 5)); break;
+            default: __builtin_amdgcn_s_waitcnt(waitcnt_vm(kScaleLoads + 6)); break;
+        }
     };
     // scales of a k block: the lane's 4 rows (one per row block) and the tile's column block
     int sa_off[4];
@@ -264,18 +296,20 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
     }
     constexpr uint32_t kSlotBytes = kSlotChunks8 * 16;
 
-    load_scales(0);
-    load_tiles(0, 0);
-    load_tiles(1, 1);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(kLoads8));  // k block 0 (and its scales) has landed; block 1 may be in flight
+    load_scales(kb_begin);
+    load_tiles(kb_begin, 0, std::false_type());
+    load_tiles(kb_begin + 1, 1, std::false_type());
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __builtin_amdgcn_s_barrier();
 
-    for (int s = 0, slot = 0; s < kblocks; ++s) {
+    auto k_loop = [&](auto all_tag) {
+    for (int s = kb_begin, slot = 0; s < kb_end; ++s) {
         float f[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) f[i] = sa_next[i] * sb_next;
         load_scales(s + 1);                           // issued before the tile loads: waiting for them later does not
-        load_tiles(s + 2, slot >= 1 ? slot - 1 : 2);  // wait for these. Slot (s + 2) % 3 was last read in k block s - 1.
+        load_tiles(s + 2, slot >= 1 ? slot - 1 : 2, all_tag);  // wait for these. Slot (s + 2) % 3 was last read in k block s - 1.
+        if (decltype(all_tag)::value || wave_active) {
         const uint32_t so = uint32_t(slot) * kSlotBytes;
         const uint32_t aa0 = a_addr[0] + so, aa1 = a_addr[1] + so, ba0 = b_addr[0] + so, ba1 = b_addr[1] + so;
         int4v_t bf[4][2], af[4][2];
@@ -330,14 +364,25 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
 #pragma unroll
             for (int v = 0; v < 4; ++v) total[3][j][v] = __builtin_fmaf(part[1][j][v], f[3], total[3][j][v]);
         }
-        // the tiles of k block s + 1 (issued one block ago) must have landed before anyone reads them; the 5 scale loads
-        // and 6 tile loads issued in this block may stay in flight
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm((SCALED ? 5 : 0) + kLoads8));
+        }
+        // the tiles of k block s + 1 (issued one block ago) must have landed before anyone reads them; the scale loads
+        // and tile loads issued in this block may stay in flight
+        wait_older_tiles(all_tag);
         __builtin_amdgcn_s_barrier();
         slot = slot == 2 ? 0 : slot + 1;
     }
+    };
+    if (a_cnt == 4) k_loop(std::true_type());
+    else k_loop(std::false_type());
     // LDS must not be released with tile loads in flight
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+
+    if (item.parts > 1) {
+        uint32_t rows_valid = 0;  // row blocks of this wave that reach into the matrix
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rows_valid |= uint32_t(m0 + wm * 64 + i * 16 < m) << i;
+        if (!gemm_k_split_fixup<kThreads8>(total, item, partials, counters, &s_last, rows_valid)) return;
+    }
 
     float alpha = 1.0f;
     if constexpr (!SCALED) {
@@ -368,10 +413,19 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
 // per-tensor scales.
 template <bool SCALED>
 static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ldb, const void *scale_a, const void *scale_b,
-                           void *c, int64_t m, int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+                           void *c, int64_t m, int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes,
+                           hipStream_t stream) {
     const int tiles_m = int(cdiv(m, kM8)), tiles_n = int(cdiv(n, kN8));
     const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
-    const int64_t grid = tiling.grid();
+    // Tail split (tiles that do not fill a round of one workgroup per CU are computed in K ranges and summed in range
+    // order by the last workgroup to arrive): at most 4 ranges of at least 4 k blocks, and only with a workspace that
+    // holds the partial tiles (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
+    GemmTail tail = make_gemm_tail(tiling, 32, 32, 4);
+    if (workspace == nullptr || workspace_bytes < kCounterBytes) tail.parts = 1;
+    while (tail.parts > 1 && (k / 128 < 4 * tail.parts ||
+                              workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * kM8 * kN8 * 4))
+        --tail.parts;
+    const int64_t grid = gemm_grid_with_tail(tiling, 32, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
     auto go = [&](auto kern) {
         static bool attr_set = false;  // one flag per kernel instantiation (the lambda is instantiated per kernel type)
@@ -381,7 +435,8 @@ static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ld
         }
         launch(kern, dim3(uint32_t(grid)), dim3(kThreads8), size_t(kLdsBytes8), stream, static_cast<const uint8_t *>(a), lda,
                static_cast<const uint8_t *>(b), ldb, static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
-               int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn);
+               int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn, tail.parts, tail.max_tiles,
+               reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
     };
     switch (out_dtype) {
         case HIDET_QMM_F32: go(gemm_fp8_kernel8<HIDET_QMM_F32, SCALED>); break;
@@ -395,16 +450,17 @@ static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ld
 // a x b^T with optional per-tensor scales on the 256 x 128, 8-wave kernel. The caller has checked: K a multiple of 128,
 // 16-byte aligned rows and pointers, N a multiple of 4, tensors below 1 GiB.
 void gemm_fp8_kernel8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
-                             int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
-    launch_kernel8<false>(a, lda, b, ldb, scale_a, scale_b, c, m, n, k, out_dtype, stream);
+                             int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
+                             hipStream_t stream) {
+    launch_kernel8<false>(a, lda, b, ldb, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
 }
 
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                            int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+                            int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     const bool fast = m * k <= (int64_t(1) << 30) && n * k <= (int64_t(1) << 30) && (k / 128) * m * 4 < (int64_t(1) << 31) &&
                       aligned(a, 16) && aligned(b, 16) && aligned(c, 16);
     if (fast) {
-        launch_kernel8<true>(a, k, b, k, scale_a, scale_b, c, m, n, k, out_dtype, stream);
+        launch_kernel8<true>(a, k, b, k, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
         return;
     }
     const int tiles_m = int(cdiv(m, kT)), tiles_n = int(n / 128);

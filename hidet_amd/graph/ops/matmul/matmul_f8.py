@@ -70,8 +70,9 @@ def _launch_f8(a2: torch.Tensor, b2: torch.Tensor, c2: torch.Tensor, scale_a, sc
     n = b2.shape[0]
     lda = a2.stride(0) if m > 1 else k
     ldb = b2.stride(0) if n > 1 else k
+    ws = ffi.workspace(a2.device)
     ffi.call('hidet_matmul_f8', a2, b2, c2, m, n, k, max(lda, k), max(ldb, k), ffi.DTYPE_CODE[c2.dtype], scale_a, scale_b,
-             ffi.current_stream(a2.device))
+             ws, ws.numel(), ffi.current_stream(a2.device))
 
 
 def _run_f8(a: torch.Tensor, b: torch.Tensor, output_dtype: torch.dtype, scale_a=None, scale_b=None) -> torch.Tensor:
@@ -129,9 +130,10 @@ class MatmulF8ScaledOperator(Operator):
         if a3.shape[0] != b3.shape[0]:
             raise ValueError('matmul_f8_scaled expects a and b with the same batch axes')
         c = torch.empty((a3.shape[0], m, n), dtype=out, device=a.device)
+        ws = ffi.workspace(a.device)
         for i in range(a3.shape[0]):
             ffi.call('hidet_matmul_f8_scaled', a3[i], b3[i], sa3[i], sb3[i], c[i], m, n, k, ffi.DTYPE_CODE[out],
-                     ffi.current_stream(a.device))
+                     ws, ws.numel(), ffi.current_stream(a.device))
         return [c.reshape(tuple(a.shape[:-2]) + (m, n))]
 
 

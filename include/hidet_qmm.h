@@ -115,14 +115,19 @@ void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *scale, int6
  * [n, k], both K-major e4m3 with row strides lda / ldb (bytes = elements); fp32 accumulation; out_dtype is the
  * element type of c (float8_e4m3, float16, bfloat16 or float32).  scale_a / scale_b are optional pointers to
  * one float32 each in device memory (per-tensor scales of the benchmark configuration); alpha is their
- * product, NULL counts as 1 (the reference's unscaled task).  No shape has to be a tile multiple. */
+ * product, NULL counts as 1 (the reference's unscaled task).  No shape has to be a tile multiple.
+ * `workspace` (optional, may be NULL; same buffer and rules as for the int8 matmul: zero-initialised once, at
+ * least hidet_qmm_min_workspace_bytes() serves every shape, one per stream) lets matrices of a few hundred
+ * rows be computed in K ranges by several workgroups per tile, summed in a fixed order; it stands in for the
+ * workspace the reference's compiled tasks request from the runtime (src/hidet/runtime/hip/context.cpp:43-57). */
 void hidet_matmul_f8(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
-                     int out_dtype, const void *scale_a, const void *scale_b, void *stream);
+                     int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
+                     void *stream);
 /* replaces MatmulF8ScaledTask (python/hidet/graph/ops/matmul/matmul_f8.py:357-454, 632-636): per K block of
  * 128, c += (sum_{k in block} a * b) * scale_a[kb, m] * scale_b[n / 128, kb]; scale_a float32 [k/128, m],
  * scale_b float32 [n/128, k/128]; a [m, k] and b [n, k] dense. */
 void hidet_matmul_f8_scaled(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                            int64_t n, int64_t k, int out_dtype, void *stream);
+                            int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

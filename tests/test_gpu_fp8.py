@@ -68,7 +68,10 @@ def test_quantize_per_tensor_every_rounding_boundary():
                                               [[1, 256], [48, 256]], [[16, 1024], [200, 1024]], [[100, 48], [36, 48]],
                                               [[300, 272], [260, 272]],
                                               # 512 tiles of 256 x 256 (two rounds of workgroups), 2 and 1 k-steps each; ragged edges
-                                              [[4096, 256], [8192, 256]], [[4096, 128], [8192, 128]], [[4000, 384], [8100, 384]]])
+                                              [[4096, 256], [8192, 256]], [[4096, 128], [8192, 128]], [[4000, 384], [8100, 384]],
+                                              # few tiles, long K: tiles computed in K ranges; short matrices in tall tiles
+                                              [[17, 4096], [2048, 4096]], [[64, 8192], [1024, 8192]], [[100, 2048], [520, 2048]],
+                                              [[200, 4096], [1152, 4096]], [[300, 2048], [1024, 2048]]])
 def test_matmul_f8_reference_recipe(a_shape, b_shape):
     # tests/operators_core/test_matmul.py:250-288: randint(-3, 3) inputs; the exact integer result is the answer
     announce('matmul_f8', a_shape, b_shape)
@@ -90,7 +93,8 @@ def test_matmul_f8_reference_recipe(a_shape, b_shape):
 
 
 @pytest.mark.parametrize('a_shape, b_shape', [[[4096, 4096], [4096, 4096]], [[2048, 256], [4096, 256]], [[100, 384], [256, 384]],
-                                              [[16384, 7168], [1536, 7168]]])
+                                              [[16384, 7168], [1536, 7168]],
+                                              [[40, 4096], [1024, 4096]], [[130, 2048], [512, 2048]], [[500, 7168], [1536, 7168]]])  # K ranges
 def test_matmul_f8_scaled_reference_recipe(a_shape, b_shape):
     # tests/operators_core/test_matmul.py:291-373: integers in [-5, 4], integer scales 1..4, bf16 output; the
     # expected value is built by pre-multiplying the scales into the operands (exact in int64)
@@ -135,6 +139,24 @@ def test_per_tensor_parity(m, k, n):
     # against the unquantized product the fp8 quantization error itself stays inside the gate
     want = a32[rows].astype(np.float64) @ b32.astype(np.float64).T
     print('max_rel_err vs unquantized', O.max_rel_err(host(got)[rows], want))
+
+
+def test_k_split_is_deterministic_and_optional():
+    announce('fp8 k split twice / without workspace')
+    from hidet_amd import ffi
+    rng = np.random.default_rng(5)
+    m, k, n = 100, 8192, 1024
+    ta = f8(rng.integers(0, 0x7F, (m, k)).astype(np.uint8))
+    tb = f8(rng.integers(0, 0x7F, (n, k)).astype(np.uint8))
+    first = host(F8.matmul_f8(ta, tb, output_dtype='float32'))
+    for _ in range(3):
+        assert np.array_equal(host(F8.matmul_f8(ta, tb, output_dtype='float32')), first)
+    # no workspace: every tile by one workgroup; same sums in a different order
+    c = torch.empty(m, n, device='cuda', dtype=torch.float32)
+    ffi.call('hidet_matmul_f8', ta, tb, c, m, n, k, k, k, ffi.DTYPE_CODE[torch.float32], None, None, None, 0,
+             ffi.current_stream(c.device))
+    ref = host(c)
+    assert O.max_rel_err(first, ref) <= 1e-5
 
 
 def test_batched_and_strided_operands():
