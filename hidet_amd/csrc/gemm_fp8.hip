@@ -232,16 +232,32 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
         voff_a[j] = ra < m ? int(int64_t(ra) * lda) + chunk * 16 : kOutside;
         voff_b[j] = rb < n ? int(int64_t(rb) * ldb) + chunk * 16 : kOutside;
     }
-    // k offsets at and past K stay inside the buffer or read zero; what they fetch is never used
-    auto load_a = [&](int step, int slot) {
+    const int steps = k / kBKB;
+    // The scalar offset is not part of the buffer's range check: a prefetch past the end of K re-reads the last step
+    // (what it fetches is never used). A tile load is kLoads instructions per wave; the loop issues them one quarter
+    // (QUARTER = 0 .. 3) at a time, one quarter per row block, so that no wave ever queues a burst of loads in front of
+    // its MFMAs (issued as a burst right behind a barrier, when all eight waves do the same, the loads cost a quarter
+    // of the kernel's time in issue stalls).
+    static_assert(kLoads % 4 == 0, "tile loads are issued in quarters");
+    auto load_a_quarter = [&](auto quarter_tag, int step, int slot) {
+        constexpr int Q = decltype(quarter_tag)::value;
+        const int soff = (step < steps ? step : steps - 1) * kBKB;
         uint4 *dst = lds + slot * kTileChunks + wave * 64;
 #pragma unroll
-        for (int j = 0; j < kLoads; ++j) buffer_load_to_lds_b128(rsrc_a, dst + j * kThr, voff_a[j], step * kBKB);
+        for (int j = Q * (kLoads / 4); j < (Q + 1) * (kLoads / 4); ++j) buffer_load_to_lds_b128(rsrc_a, dst + j * kThr, voff_a[j], soff);
     };
-    auto load_b = [&](int step, int slot) {
+    auto load_b_quarter = [&](auto quarter_tag, int step, int slot) {
+        constexpr int Q = decltype(quarter_tag)::value;
+        const int soff = (step < steps ? step : steps - 1) * kBKB;
         uint4 *dst = lds + (kASlots + slot) * kTileChunks + wave * 64;
 #pragma unroll
-        for (int j = 0; j < kLoads; ++j) buffer_load_to_lds_b128(rsrc_b, dst + j * kThr, voff_b[j], step * kBKB);
+        for (int j = Q * (kLoads / 4); j < (Q + 1) * (kLoads / 4); ++j) buffer_load_to_lds_b128(rsrc_b, dst + j * kThr, voff_b[j], soff);
+    };
+    auto load_a = [&](int step, int slot) {
+        static_for<0, 4>([&](auto qt) { load_a_quarter(qt, step, slot); });
+    };
+    auto load_b = [&](int step, int slot) {
+        static_for<0, 4>([&](auto qt) { load_b_quarter(qt, step, slot); });
     };
 
     // LDS byte addresses of this lane's two 16-byte fragment halves in block 0 of its wave, slot 0 of each ring;
@@ -257,13 +273,15 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
     }
     constexpr uint32_t kSlotBytes = kTileChunks * 16;
 
-    const int steps = k / kBKB;
+    // Issue order of the tile loads (A ring: 3 slots, B ring: 2): the A tile of step s + 3 goes out one quarter each in
+    // row block 7 of step s (behind barrier L, which frees its slot) and row blocks 0, 1, 2 of step s + 1; the B tile of
+    // step s + 2 one quarter each in row blocks 3 .. 6 of step s (behind barrier P, which frees its slot).
     load_a(0, 0);
     load_b(0, 0);
     load_a(1, 1);
     load_b(1, 1);
-    load_a(2, 2);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(3 * kLoads));
+    load_a_quarter(std::integral_constant<int, 0>(), 2, 2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * kLoads + kLoads / 4));
     __builtin_amdgcn_s_barrier();
 
     int4v_t bf[NB][2], af[3][2];
@@ -284,12 +302,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
     for (int s = 0; s < steps; ++s) {
         const uint32_t aa0 = a_addr[0] + uint32_t(a_slot) * kSlotBytes, aa1 = a_addr[1] + uint32_t(a_slot) * kSlotBytes;
         const int a_next = a_slot == kASlots - 1 ? 0 : a_slot + 1, b_next = b_slot ^ 1;
+        const int a_prev = a_slot == 0 ? kASlots - 1 : a_slot - 1;  // freed by barrier L of the previous step: takes step s + 2
 
         // ---- row block 0: the reads outstanding are a0, b0 .. b(NB-1) of this step (in either order of a0 and b0);
         // the B fragments arrive one by one, a1 is requested behind the first MFMA
         lds_wait_keep_newer<2 * (NB - 1)>(bf[0][0], bf[0][1]);
         lds_wait_keep_newer<2 * (NB - 1)>(af[0][0], af[0][1]);
         mfma_fp8_k128v(bf[0][0], bf[0][1], af[0][0], af[0][1], acc[0][0], unit_scales);
+        load_a_quarter(std::integral_constant<int, 1>(), s + 2, a_prev);
         af[1][0] = lds_read_b128_early<1 * 2048>(aa0);
         af[1][1] = lds_read_b128_early<1 * 2048>(aa1);
         static_for<1, NB>([&](auto jt) {
@@ -300,7 +320,6 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
         });
         // barrier P: every wave holds all B fragments of this step, so its B slot can take step s + 2
         __builtin_amdgcn_s_barrier();
-        load_b(s + 2, b_slot);
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- row blocks 1 .. 6
@@ -309,8 +328,11 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
             af[(I + 1) % 3][0] = lds_read_b128_early<(I + 1) * 2048>(aa0);
             af[(I + 1) % 3][1] = lds_read_b128_early<(I + 1) * 2048>(aa1);
             lds_wait_keep_newer<2>(af[I % 3][0], af[I % 3][1]);
+            mfma_fp8_k128v(bf[0][0], bf[0][1], af[I % 3][0], af[I % 3][1], acc[I][0], unit_scales);
+            if constexpr (I <= 2) load_a_quarter(std::integral_constant<int, I + 1>(), s + 2, a_prev);
+            else load_b_quarter(std::integral_constant<int, I - 3>(), s + 2, b_slot);
 #pragma unroll
-            for (int j = 0; j < NB; ++j) mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j], unit_scales);
+            for (int j = 1; j < NB; ++j) mfma_fp8_k128v(bf[j][0], bf[j][1], af[I % 3][0], af[I % 3][1], acc[I][j], unit_scales);
             __builtin_amdgcn_sched_barrier(0);
         });
 
@@ -320,7 +342,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
         lds_wait_keep_newer<0>(af[1][0], af[1][1]);
         __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * kLoads));
         __builtin_amdgcn_s_barrier();
-        load_a(s + 3, a_slot);
+        load_a_quarter(std::integral_constant<int, 0>(), s + 3, a_slot);
         __builtin_amdgcn_sched_barrier(0);
         {
             const uint32_t na0 = a_addr[0] + uint32_t(a_next) * kSlotBytes, na1 = a_addr[1] + uint32_t(a_next) * kSlotBytes;
