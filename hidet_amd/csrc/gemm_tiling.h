@@ -65,7 +65,7 @@ struct GemmRegion {
     int row_begin, col_begin, rows, cols;
 };
 
-__device__ __forceinline__ GemmRegion gemm_region_of_xcd(int tiles_m, int tiles_n, int xm, int xn, int xcd) {
+__host__ __device__ __forceinline__ GemmRegion gemm_region_of_xcd(int tiles_m, int tiles_n, int xm, int xn, int xcd) {
     const int xr = xcd / xn, xc = xcd % xn;
     const int r_begin = (tiles_m * xr) / xm, r_end = (tiles_m * (xr + 1)) / xm;
     const int c_begin = (tiles_n * xc) / xn, c_end = (tiles_n * (xc + 1)) / xn;
@@ -73,7 +73,7 @@ __device__ __forceinline__ GemmRegion gemm_region_of_xcd(int tiles_m, int tiles_
 }
 
 // Tile (row, column) number `local` of a region in panel order; false past the end of the region.
-__device__ __forceinline__ bool gemm_tile_of_region(const GemmRegion &reg, int local, int *tile_m, int *tile_n) {
+__host__ __device__ __forceinline__ bool gemm_tile_of_region(const GemmRegion &reg, int local, int *tile_m, int *tile_n) {
     const int rr = reg.rows, rc = reg.cols;
     if (local >= rr * rc) return false;
     const int full_panels = rc / kPanelCols;
@@ -95,7 +95,7 @@ __device__ __forceinline__ bool gemm_tile_of_region(const GemmRegion &reg, int l
 
 // Tile (row, column) of this workgroup; false when it has none (its XCD's region is smaller than the largest).
 __device__ __forceinline__ bool gemm_tile_of_block(int tiles_m, int tiles_n, int xm, int xn, int *tile_m, int *tile_n) {
-    const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, blockIdx.x & 7);
+    const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, blockIdx.x & 7);  // workgroup b runs on XCD b % 8
     return gemm_tile_of_region(reg, blockIdx.x >> 3, tile_m, tile_n);
 }
 
@@ -136,12 +136,14 @@ struct GemmWorkItem {
     int tile_m, tile_n, part, parts, slot;
 };
 
-__device__ __forceinline__ bool gemm_work_item(int tiles_m, int tiles_n, int xm, int xn, int concurrent, int tail_parts,
-                                               int tail_stride, GemmWorkItem *item) {
-    const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, blockIdx.x & 7);
+// (Workgroup `block` of the launch; a pure function so that the host can enumerate a launch, as the tests do.)
+__host__ __device__ __forceinline__ bool gemm_work_item_of_block(int block, int tiles_m, int tiles_n, int xm, int xn,
+                                                                 int concurrent, int tail_parts, int tail_stride,
+                                                                 GemmWorkItem *item) {
+    const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, block & 7);
     const int region_tiles = reg.rows * reg.cols;
     const int whole = tail_parts > 1 ? (region_tiles / concurrent) * concurrent : region_tiles;
-    int local = blockIdx.x >> 3;
+    int local = block >> 3;
     item->part = 0;
     item->parts = 1;
     item->slot = 0;
@@ -150,9 +152,14 @@ __device__ __forceinline__ bool gemm_work_item(int tiles_m, int tiles_n, int xm,
         local = whole + j / tail_parts;
         item->part = j % tail_parts;
         item->parts = tail_parts;
-        item->slot = (blockIdx.x & 7) * tail_stride + j / tail_parts;
+        item->slot = (block & 7) * tail_stride + j / tail_parts;
     }
     return gemm_tile_of_region(reg, local, &item->tile_m, &item->tile_n);
+}
+
+__device__ __forceinline__ bool gemm_work_item(int tiles_m, int tiles_n, int xm, int xn, int concurrent, int tail_parts,
+                                               int tail_stride, GemmWorkItem *item) {
+    return gemm_work_item_of_block(int(blockIdx.x), tiles_m, tiles_n, xm, xn, concurrent, tail_parts, tail_stride, item);
 }
 
 // Fix-up of a tile computed in K ranges by item.parts workgroups of THREADS threads, each holding R x T float4

@@ -1,0 +1,61 @@
+// Host-side enumeration of GEMM launches: every tile of the output must be computed exactly once (all of its K ranges,
+// each by one workgroup), and the tiles that are split must get distinct fix-up slots inside the planned storage.
+// Built and run by tests/test_tiling.py; exits non-zero with a message on the first violation.
+#include <cstdio>
+#include <vector>
+
+#include "gemm_tiling.h"
+
+using namespace qmm;
+
+static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_parts, bool tile_only) {
+    const GemmTiling t = make_gemm_tiling(tiles_m, tiles_n, concurrent);
+    if (t.xm * t.xn != 8) return std::printf("tiling %dx%d: %d x %d regions\n", tiles_m, tiles_n, t.xm, t.xn), 1;
+    GemmTail tail = make_gemm_tail(t, concurrent, fill, max_parts);
+    if (tile_only) tail = GemmTail{1, 0, t.grid()};
+    const long long grid = gemm_grid_with_tail(t, concurrent, tail);
+    std::vector<int> seen(size_t(tiles_m) * tiles_n * max_parts, 0), parts_of(size_t(tiles_m) * tiles_n, 0);
+    std::vector<int> slot_owner(size_t(8) * (tail.max_tiles > 0 ? tail.max_tiles : 1), -1);
+    for (long long b = 0; b < grid; ++b) {
+        GemmWorkItem it;
+        if (!gemm_work_item_of_block(int(b), tiles_m, tiles_n, t.xm, t.xn, concurrent, tail.parts, tail.max_tiles, &it)) continue;
+        if (it.tile_m < 0 || it.tile_m >= tiles_m || it.tile_n < 0 || it.tile_n >= tiles_n || it.part < 0 || it.part >= it.parts ||
+            it.parts > max_parts)
+            return std::printf("%dx%d c%d: block %lld -> tile (%d, %d) part %d/%d\n", tiles_m, tiles_n, concurrent, b, it.tile_m,
+                               it.tile_n, it.part, it.parts), 1;
+        const size_t tile = size_t(it.tile_m) * tiles_n + it.tile_n;
+        if (parts_of[tile] != 0 && parts_of[tile] != it.parts)
+            return std::printf("%dx%d c%d: tile %zu seen with %d and %d parts\n", tiles_m, tiles_n, concurrent, tile, parts_of[tile], it.parts), 1;
+        parts_of[tile] = it.parts;
+        if (seen[tile * max_parts + it.part]++)
+            return std::printf("%dx%d c%d: tile %zu part %d computed twice\n", tiles_m, tiles_n, concurrent, tile, it.part), 1;
+        if (it.parts > 1) {
+            if (it.slot < 0 || it.slot >= int(slot_owner.size()))
+                return std::printf("%dx%d c%d: slot %d outside %zu\n", tiles_m, tiles_n, concurrent, it.slot, slot_owner.size()), 1;
+            if (slot_owner[it.slot] >= 0 && slot_owner[it.slot] != int(tile))
+                return std::printf("%dx%d c%d: slot %d shared by tiles %d and %zu\n", tiles_m, tiles_n, concurrent, it.slot, slot_owner[it.slot], tile), 1;
+            slot_owner[it.slot] = int(tile);
+        }
+    }
+    for (size_t tile = 0; tile < parts_of.size(); ++tile) {
+        if (parts_of[tile] == 0) return std::printf("%dx%d c%d: tile %zu never computed\n", tiles_m, tiles_n, concurrent, tile), 1;
+        for (int p = 0; p < parts_of[tile]; ++p)
+            if (seen[tile * max_parts + p] != 1)
+                return std::printf("%dx%d c%d: tile %zu part %d missing\n", tiles_m, tiles_n, concurrent, tile, p), 1;
+    }
+    return 0;
+}
+
+int main() {
+    long long n = 0;
+    const int cfgs[][3] = {{32, 32, 4}, {32, 32, 8}, {64, 64, 4}, {64, 32, 4}};  // concurrent, fill, max_parts of the launchers
+    for (const auto &c : cfgs)
+        for (int tm = 1; tm <= 70; tm += (tm < 20 ? 1 : 7))
+            for (int tn = 1; tn <= 130; tn += (tn < 50 ? 1 : 9)) {
+                if (check(tm, tn, c[0], c[1], c[2], false)) return 1;
+                if (check(tm, tn, c[0], c[1], c[2], true)) return 1;
+                n += 2;
+            }
+    std::printf("ok %lld launches\n", n);
+    return 0;
+}
