@@ -22,12 +22,16 @@ __device__ __forceinline__ uint16_t skinny_to_out<uint16_t>(float v) { return f3
 
 // Workgroup -> (column tile, K split).  Workgroups are dealt round-robin to the 8 XCDs: every K split
 // of a column tile gets the same residue mod 8, so the partial tiles of a column tile meet in one L2.
-__device__ __forceinline__ bool skinny_tile_of_block(int splits, int tiles, int *tile, int *split) {
-    const int bid = blockIdx.x;
+// (skinny_tile_of: workgroup `bid` of a launch of cdiv(tiles, 8) * 8 * splits workgroups; a pure function so that the
+// host can enumerate a launch, as the tests do.)
+__host__ __device__ __forceinline__ bool skinny_tile_of(int bid, int splits, int tiles, int *tile, int *split) {
     const int rest = bid >> 3;
     *split = rest % splits;
     *tile = (rest / splits) * 8 + (bid & 7);
     return *tile < tiles;
+}
+__device__ __forceinline__ bool skinny_tile_of_block(int splits, int tiles, int *tile, int *split) {
+    return skinny_tile_of(int(blockIdx.x), splits, tiles, tile, split);
 }
 
 // res[t][v] is this lane's partial sum for output row 4 * (lane / 16) + v and column

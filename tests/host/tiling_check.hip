@@ -1,10 +1,11 @@
-// Host-side enumeration of GEMM launches: every tile of the output must be computed exactly once (all of its K ranges,
-// each by one workgroup), and the tiles that are split must get distinct fix-up slots inside the planned storage.
+// Host-side enumeration of launches: every tile of the output must be computed exactly once (all of its K ranges or
+// slices, each by one workgroup), and GEMM tiles that are split must get distinct fix-up slots inside the planned storage.
 // Built and run by tests/test_tiling.py; exits non-zero with a message on the first violation.
 #include <cstdio>
 #include <vector>
 
 #include "gemm_tiling.h"
+#include "skinny_common.h"
 
 using namespace qmm;
 
@@ -46,8 +47,36 @@ static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_par
     return 0;
 }
 
+// Bandwidth-bound kernels: K is cut into `splits` slices of rows_per_block rows (whole multiples of the granule) that
+// cover K exactly once, and every (column tile, slice) pair belongs to exactly one workgroup.
+static int check_skinny(long long k, long long ncols, int slice_rows, int hint, int granule) {
+    int rpb = 0, splits = 0, tiles = 0;
+    skinny_plan(k, ncols, slice_rows, hint, granule, &rpb, &splits, &tiles);
+    if (rpb <= 0 || rpb % granule != 0 || splits < 1 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
+        tiles != int((ncols + kSkinnyTileN - 1) / kSkinnyTileN))
+        return std::printf("skinny k=%lld n=%lld hint=%d: rows %d x %d splits, %d tiles\n", k, ncols, hint, rpb, splits, tiles), 1;
+    std::vector<int> seen(size_t(tiles) * splits, 0);
+    const int grid = ((tiles + 7) / 8) * 8 * splits;
+    for (int b = 0; b < grid; ++b) {
+        int tile, split;
+        if (!skinny_tile_of(b, splits, tiles, &tile, &split)) continue;
+        if (tile < 0 || split < 0 || split >= splits || seen[size_t(tile) * splits + split]++)
+            return std::printf("skinny k=%lld n=%lld: block %d -> tile %d split %d\n", k, ncols, b, tile, split), 1;
+    }
+    for (int v : seen)
+        if (v != 1) return std::printf("skinny k=%lld n=%lld: a slice has no workgroup\n", k, ncols), 1;
+    return 0;
+}
+
 int main() {
     long long n = 0;
+    for (long long k : {32LL, 96LL, 128LL, 1000LL, 4096LL, 11008LL, 8192LL, 28672LL})
+        for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL})
+            for (int hint : {0, 1, 3, 8, 64})
+                for (int cfg = 0; cfg < 3; ++cfg) {
+                    if (check_skinny(k, nc, cfg == 1 ? 768 : 512, hint, cfg == 2 ? 256 : 128)) return 1;
+                    ++n;
+                }
     const int cfgs[][3] = {{32, 32, 4}, {32, 32, 8}, {64, 64, 4}, {64, 32, 4}};  // concurrent, fill, max_parts of the launchers
     for (const auto &c : cfgs)
         for (int tm = 1; tm <= 70; tm += (tm < 20 ? 1 : 7))

@@ -1,5 +1,6 @@
-"""Host logic of the GEMM launch plans (2D XCD regions, panels, K split of tail tiles): a small host program
-enumerates every workgroup of many launches and checks that each output tile is computed exactly once."""
+"""Host logic of the launch plans (GEMMs: 2D XCD regions, panels, K split of tail tiles; bandwidth-bound kernels: K
+slices x column tiles): a small host program enumerates every workgroup of many launches and checks that each output
+tile, and each K range or slice of it, is computed exactly once."""
 import os
 import shutil
 import subprocess
