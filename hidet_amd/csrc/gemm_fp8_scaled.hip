@@ -253,6 +253,11 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
             if (decltype(all_tag)::value || j >= 4 || j < a_cnt)
                 buffer_load_to_lds_b128(j < 4 ? rsrc_a : rsrc_b, dst + j * kThreads8, voff[j], kbc * 128);
     };
+    auto load_tile_one = [&](auto j_tag, int kb, int slot) {  // one of the kLoads8 instructions of load_tiles, full tiles
+        constexpr int J = decltype(j_tag)::value;
+        const int kbc = kb < kblocks ? kb : kblocks - 1;
+        buffer_load_to_lds_b128(J < 4 ? rsrc_a : rsrc_b, lds + slot * kSlotChunks8 + wave * 64 + J * kThreads8, voff[J], kbc * 128);
+    };
     auto wait_older_tiles = [&](auto all_tag) {  // everything but the loads of the last load_scales + load_tiles has landed
         constexpr int kScaleLoads = SCALED ? 5 : 0;
         if (decltype(all_tag)::value) {
@@ -308,7 +313,17 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
 #pragma unroll
         for (int i = 0; i < 4; ++i) f[i] = sa_next[i] * sb_next;
         load_scales(s + 1);                           // issued before the tile loads: waiting for them later does not
-        load_tiles(s + 2, slot >= 1 ? slot - 1 : 2, all_tag);  // wait for these. Slot (s + 2) % 3 was last read in k block s - 1.
+        // wait for these. Slot (s + 2) % 3 was last read in k block s - 1. Full tiles issue the six load instructions two,
+        // two, one and one at a time between the row blocks instead of in one burst behind the barrier (every wave of the
+        // workgroup would queue its burst at the same moment, in front of its MFMAs).
+        constexpr bool kSpread = decltype(all_tag)::value;
+        const int slot_in = slot >= 1 ? slot - 1 : 2;
+        if constexpr (kSpread) {
+            load_tile_one(std::integral_constant<int, 0>(), s + 2, slot_in);
+            load_tile_one(std::integral_constant<int, 1>(), s + 2, slot_in);
+        } else {
+            load_tiles(s + 2, slot_in, all_tag);
+        }
         if (decltype(all_tag)::value || wave_active) {
         const uint32_t so = uint32_t(slot) * kSlotBytes;
         const uint32_t aa0 = a_addr[0] + so, aa1 = a_addr[1] + so, ba0 = b_addr[0] + so, ba1 = b_addr[1] + so;
@@ -341,12 +356,17 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
         mm(part[0][2], total[0][2], bf[2][0], bf[2][1], af[0][0], af[0][1]);
         lds_wait_keep_newer<6>(bf[3][0], bf[3][1]);
         mm(part[0][3], total[0][3], bf[3][0], bf[3][1], af[0][0], af[0][1]);
+        if constexpr (kSpread) {
+            load_tile_one(std::integral_constant<int, 2>(), s + 2, slot_in);
+            load_tile_one(std::integral_constant<int, 3>(), s + 2, slot_in);
+        }
         __builtin_amdgcn_sched_barrier(0);
         auto row_block = [&](auto i_tag) {  // MFMAs of row block I, then the fold of row block I - 1 behind them
             constexpr int I = decltype(i_tag)::value;
             lds_wait_keep_newer<2 * (3 - I)>(af[I][0], af[I][1]);
 #pragma unroll
             for (int j = 0; j < 4; ++j) mm(part[I & 1][j], total[I][j], bf[j][0], bf[j][1], af[I][0], af[I][1]);
+            if constexpr (kSpread && I <= 2) load_tile_one(std::integral_constant<int, 3 + I>(), s + 2, slot_in);
             if constexpr (SCALED) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
