@@ -5,6 +5,8 @@
 
 #include <cstdint>
 #include <exception>
+#include <mutex>
+#include <set>
 #include <sstream>
 #include <string>
 
@@ -92,6 +94,19 @@ inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem
         hipLaunchKernelGGL(kernel, grid, block, shmem, stream, static_cast<KArgs>(args)...);
     }
     QMM_HIP(hipGetLastError());
+}
+
+// A kernel that uses more than 64 KiB of dynamic LDS has to be told so once per device before its first launch there.
+inline void allow_dynamic_lds(const void *kernel, int bytes) {
+    if (bytes <= 65536) return;
+    static std::mutex mu;
+    static std::set<std::pair<const void *, int>> done;
+    int device = 0;
+    QMM_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> guard(mu);
+    if (done.count({kernel, device})) return;
+    QMM_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    done.insert({kernel, device});
 }
 
 // Helper kernels (fills, conversions) never consume the timing slot.

@@ -445,12 +445,6 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
         const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
         const int64_t grid = tiling.grid();
         QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-        static bool attr_set = false;  // one flag per output type (the lambda is instantiated per type)
-        if (!attr_set) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_staged_kernel<OUT>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
-            attr_set = true;
-        }
         const bool fast = (k % kBKB == 0) && (m - 1) * lda + k <= (int64_t(1) << 30) &&
                           (n - 1) * ldb + k <= (int64_t(1) << 30);
         if (fast) {
@@ -463,16 +457,12 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
                 gemm_fp8_kernel8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, workspace, workspace_bytes, stream);
                 return;
             }
-            static bool fast_attr_set = false;
-            if (!fast_attr_set) {
-                QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp8_kernel<OUT, 8>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, kFastLdsBytes));
-                fast_attr_set = true;
-            }
+            allow_dynamic_lds(reinterpret_cast<const void *>(gemm_fp8_kernel<OUT, 8>), kFastLdsBytes);
             launch(gemm_fp8_kernel<OUT, 8>, dim3(uint32_t(grid)), dim3(512), size_t(kFastLdsBytes), stream, ap, lda, bp, ldb, c,
                    int(m), int(n), int(k), sa, sb, tiles_m, tiles_n, tiling.xm, tiling.xn);
             return;
         }
+        allow_dynamic_lds(reinterpret_cast<const void *>(gemm_fp8_staged_kernel<OUT>), kLdsBytes);
         launch(gemm_fp8_staged_kernel<OUT>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kLdsBytes), stream, ap, lda, bp, ldb, c,
                int(m), int(n), int(k), sa, sb, tiles_m, tiles_n, tiling.xm, tiling.xn);
     });

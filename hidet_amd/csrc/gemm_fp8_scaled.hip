@@ -448,11 +448,7 @@ static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ld
     const int64_t grid = gemm_grid_with_tail(tiling, 32, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
     auto go = [&](auto kern) {
-        static bool attr_set = false;  // one flag per kernel instantiation (the lambda is instantiated per kernel type)
-        if (!attr_set) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes8));
-            attr_set = true;
-        }
+        allow_dynamic_lds(reinterpret_cast<const void *>(kern), kLdsBytes8);
         launch(kern, dim3(uint32_t(grid)), dim3(kThreads8), size_t(kLdsBytes8), stream, static_cast<const uint8_t *>(a), lda,
                static_cast<const uint8_t *>(b), ldb, static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
                int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn, tail.parts, tail.max_tiles,

@@ -458,14 +458,7 @@ void launch_cfg16(const void *a, const void *w, const void *scales, void *c, int
         --tail.parts;
     const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-    if (Cfg::kLdsBytes > 65536) {
-        static bool attr_set = false;
-        if (!attr_set) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a16_kernel16<DT, RB, WM, WN, MIN_BLOCKS>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
-            attr_set = true;
-        }
-    }
+    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w4a16_kernel16<DT, RB, WM, WN, MIN_BLOCKS>), Cfg::kLdsBytes);
     launch(gemm_w4a16_kernel16<DT, RB, WM, WN, MIN_BLOCKS>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes),
            stream, static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
            static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,
@@ -830,12 +823,7 @@ void launch_lds(const void *a, const void *w, const void *scales, void *c, int64
         --tail.parts;
     const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-    static bool attr_set = false;
-    if (!attr_set) {
-        QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a16_lds_kernel<DT>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
-        attr_set = true;
-    }
+    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w4a16_lds_kernel<DT>), Cfg::kLdsBytes);
     launch(gemm_w4a16_lds_kernel<DT>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
            static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,

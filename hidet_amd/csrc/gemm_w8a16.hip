@@ -273,14 +273,7 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     static_assert(8 * kConcurrent * 4 <= kCounterBytes, "one counter per tail tile");
     const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-    if (Cfg::kLdsBytes > 65536) {
-        static bool attr_set = false;
-        if (!attr_set) {
-            QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::kLdsBytes));
-            attr_set = true;
-        }
-    }
+    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>), Cfg::kLdsBytes);
     launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale),
            static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent, tail.parts, tail.max_tiles,

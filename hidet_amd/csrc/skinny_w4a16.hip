@@ -225,7 +225,7 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
         uint32_t *counters = static_cast<uint32_t *>(workspace);
         const size_t shmem = skinny_lds_bytes(mt);
         auto go = [&](auto kern) {
-            if (shmem > 65536) QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(shmem)));
+            if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16)));  // the most any m needs
             launch(kern, dim3(grid), dim3(256), shmem, stream, ap0 + m0 * lda, lda, wp, sp, cp0 + m0 * n, mt, int(k), int(n),
                    group, rpb, splits, tiles, partials, counters);
         };

@@ -154,7 +154,7 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
         _Float16 *cp = static_cast<_Float16 *>(c) + m0 * n;
         const size_t shmem = skinny_lds_bytes(mt);
         auto go = [&](auto kern) {
-            if (shmem > 65536) QMM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(shmem)));
+            if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16)));  // the most any m needs
             launch(kern, dim3(grid), dim3(256), shmem, stream, ap, lda, static_cast<const int8_t *>(w),
                    static_cast<const _Float16 *>(scale), cp, mt, int(k), int(n), rpb, splits, tiles, partials, counters);
         };
