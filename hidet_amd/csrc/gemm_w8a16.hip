@@ -110,7 +110,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
     auto load_a = [&](int st, int slot) {
 #pragma unroll
         for (int j = 0; j < kAChunksActive; ++j)
-            buffer_load_to_lds_b128(rsrc_a, lds + slot * Cfg::kBM * 8 + j * Cfg::kThreads + wave * 64, a_off[j], st * (kBK * 2));
+            buffer_load_to_lds_b128(rsrc_a, lds + slot * Cfg::kBM * 8 + j * Cfg::kThreads + wave * 64, a_off[j],
+                                    (st < stages ? st : stages - 1) * (kBK * 2));  // the scalar offset is not range-checked
     };
     auto load_w = [&](int st, int q, uint32_t (&dst)[8]) {
         const int soff = ((st < stages ? st : stages - 1) * kBK + q * 32) * n;
