@@ -286,6 +286,16 @@ def main():
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ad, ws[r % RING].view(N, K), sd, cd, 1, N, K, N, 0,
                                       work, work.numel(), sptr), 48, 16)
     others['w8a16_gemv_down_proj_k11008_n4096'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * K)
+    # the same GEMV kernel on a matrix five times the size (not a benchmark configuration: it shows how much of the headline
+    # figure is the fixed cost of one launch and one cross-workgroup exchange)
+    wl = [torch.randint(-127, 128, (8192, 28672), device=device, dtype=torch.int8) for _ in range(3)]  # 3 x 235 MB > LLC
+    al = torch.randn((1, 8192), generator=g, device=device, dtype=torch.float32).to(torch.float16)
+    sl = torch.cat([ss[0], ss[1], ss[2]])[:28672].contiguous()
+    cl = torch.empty((1, 28672), dtype=torch.float16, device=device)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', al, wl[r % 3], sl, cl, 1, 8192, 28672, 8192, 0,
+                                      work, work.numel(), sptr), 24, 6)
+    others['w8a16_gemv_k8192_n28672_not_a_baseline_config'] = hbm_entry(us, 8192 * 28672 + 2 * 28672 + 2 * 8192 + 2 * 28672)
+    del wl
     # W8A16 prefill, attention QKV shape [2048, 4096] x [4096, 12288]
     wq = [torch.randint(-127, 128, (K, 12288), device=device, dtype=torch.int8) for _ in range(4)]
     sq = torch.cat([ss[0], ss[1]])[:12288].contiguous()
