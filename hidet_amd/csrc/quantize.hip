@@ -165,6 +165,99 @@ __global__ __launch_bounds__(256) void quantize4_kernel(const void *__restrict__
     }
 }
 
+// Same arithmetic for [outer, R, inner] with inner a multiple of 4, laid out so that nothing is recomputed per element:
+// grid (ceil(inner / 256), ceil(R / kQuantRows), outer), 256 threads = 4 row lanes x 64 column quads. A thread keeps its
+// four columns, works out their four scales once (the element-per-thread kernels divide amax / qmax again for every
+// element and pay two 64-bit index divisions per thread) and walks kQuantRows / 4 rows with 16-byte loads.
+constexpr int kQuantRows = 32;
+template <int DT, int QT>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const void *__restrict__ w, const uint32_t *__restrict__ amax_bits,
+                                                            void *__restrict__ q, void *__restrict__ scale, int64_t R,
+                                                            int64_t inner4) {
+    const float qmax = QT == HIDET_QMM_I8 ? 127.0f : 32767.0f;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int64_t c4 = int64_t(blockIdx.x) * 64 + tx;
+    if (c4 >= inner4) return;
+    const int64_t o = blockIdx.z;
+    const int64_t sidx = (o * inner4 + c4) * 4;
+    const uint4 ab = *reinterpret_cast<const uint4 *>(amax_bits + sidx);
+    const uint32_t abits[4] = {ab.x, ab.y, ab.z, ab.w};
+    float s[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] = round_to<DT>(__uint_as_float(abits[e]) / qmax);
+    if (blockIdx.y == 0 && ty == 0) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) store_from_f32<DT>(scale, sidx + e, s[e]);
+    }
+    const int64_t r_end = min(R, (int64_t(blockIdx.y) + 1) * kQuantRows);
+    for (int64_t r = int64_t(blockIdx.y) * kQuantRows + ty; r < r_end; r += 4) {
+        const int64_t i4 = (o * R + r) * inner4 + c4;
+        float x[4], code[4];
+        load4_as_f32<DT>(w, i4, x);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) code[e] = s[e] != 0.0f ? roundf(round_to<DT>(x[e] / s[e])) : 0.0f;
+        if (QT == HIDET_QMM_I8) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) packed |= uint32_t(uint8_t(int8_t(fminf(fmaxf(code[e], -128.0f), 127.0f)))) << (8 * e);
+            static_cast<uint32_t *>(q)[i4] = packed;
+        } else {
+            uint32_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = uint32_t(uint16_t(int16_t(fminf(fmaxf(code[e], -32768.0f), 32767.0f))));
+            static_cast<uint2 *>(q)[i4] = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+    }
+}
+
+// inner == 1 (one scale per row, e.g. an embedding table): one workgroup per row keeps the whole row in registers
+// between the amax pass and the quantization, so the tensor is read once. Rows of up to 256 * 4 * NV elements, a
+// multiple of 4, 16-byte aligned. Same arithmetic as above.
+template <int DT, int QT, int NV>
+__global__ __launch_bounds__(256) void quantize_row_fused_kernel(const void *__restrict__ w, void *__restrict__ q,
+                                                                 void *__restrict__ scale, int64_t R4) {
+    __shared__ float red[4];
+    const float qmax = QT == HIDET_QMM_I8 ? 127.0f : 32767.0f;
+    const int tid = threadIdx.x;
+    const int64_t base4 = int64_t(blockIdx.x) * R4;
+    float x[NV][4];
+    float m = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t j = int64_t(v) * 256 + tid;
+        x[v][0] = x[v][1] = x[v][2] = x[v][3] = 0.0f;
+        if (j < R4) load4_as_f32<DT>(w, base4 + j, x[v]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) m = fmaxf(m, fabsf(x[v][e]));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const float s = round_to<DT>(m / qmax);
+    if (tid == 0) store_from_f32<DT>(scale, blockIdx.x, s);
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t j = int64_t(v) * 256 + tid;
+        if (j >= R4) continue;
+        float code[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) code[e] = s != 0.0f ? roundf(round_to<DT>(x[v][e] / s)) : 0.0f;
+        if (QT == HIDET_QMM_I8) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) packed |= uint32_t(uint8_t(int8_t(fminf(fmaxf(code[e], -128.0f), 127.0f)))) << (8 * e);
+            static_cast<uint32_t *>(q)[base4 + j] = packed;
+        } else {
+            uint32_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = uint32_t(uint16_t(int16_t(fminf(fmaxf(code[e], -32768.0f), 32767.0f))));
+            static_cast<uint2 *>(q)[base4 + j] = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+    }
+}
+
 template <int QT, int ST>
 __global__ __launch_bounds__(256) void dequantize_kernel(const void *__restrict__ q, const void *__restrict__ scale,
                                                          void *__restrict__ w, int64_t R, int64_t inner, int64_t total) {
@@ -353,6 +446,18 @@ HIDET_API void hidet_symmetric_quantize(const void *w, void *wq, void *scale, in
     uint32_t *amax_bits = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kCounterBytes);
     dispatch_float(w_dtype, [&](auto dt) {
         constexpr int DT = decltype(dt)::value;
+        {
+            // rows that fit a workgroup's registers: one pass
+            const int esize0 = DT == HIDET_QMM_F32 ? 4 : 2, qsize0 = q_dtype == HIDET_QMM_I8 ? 1 : 2;
+            if (inner == 1 && reduce > 0 && reduce % 4 == 0 && reduce <= 256 * 4 * 16 && outer < (int64_t(1) << 31) &&
+                aligned(w, 4 * esize0) && aligned(wq, 4 * qsize0) && aligned(scale, esize0)) {
+                auto go = [&](auto kern) { launch(kern, dim3(uint32_t(outer)), dim3(256), 0, stream, w, wq, scale, reduce / 4); };
+                const bool small = reduce <= 256 * 4 * 4;
+                if (q_dtype == HIDET_QMM_I8) small ? go(quantize_row_fused_kernel<DT, HIDET_QMM_I8, 4>) : go(quantize_row_fused_kernel<DT, HIDET_QMM_I8, 16>);
+                else small ? go(quantize_row_fused_kernel<DT, HIDET_QMM_I16, 4>) : go(quantize_row_fused_kernel<DT, HIDET_QMM_I16, 16>);
+                return;
+            }
+        }
         if (reduce == 0) {
             launch_aux(fill_u32_kernel, dim3(cdiv(nscale, 256)), dim3(256), 0, stream, amax_bits, nscale, 0u);
         } else if (inner == 1) {
@@ -373,6 +478,15 @@ HIDET_API void hidet_symmetric_quantize(const void *w, void *wq, void *scale, in
         const int esize = DT == HIDET_QMM_F32 ? 4 : 2, qsize = q_dtype == HIDET_QMM_I8 ? 1 : 2;
         const bool vec_ok = aligned(w, 4 * esize) && aligned(wq, 4 * qsize) && aligned(scale, esize);
         if (vec_ok && inner % 4 == 0) {
+            const int64_t row_blocks = cdiv(reduce, kQuantRows);
+            if (row_blocks <= 65535 && outer <= 65535) {
+                const dim3 grid(uint32_t(cdiv(inner / 4, 64)), uint32_t(row_blocks), uint32_t(outer));
+                if (q_dtype == HIDET_QMM_I8)
+                    launch(quantize_rows_kernel<DT, HIDET_QMM_I8>, grid, dim3(256), 0, stream, w, amax_bits, wq, scale, reduce, inner / 4);
+                else
+                    launch(quantize_rows_kernel<DT, HIDET_QMM_I16>, grid, dim3(256), 0, stream, w, amax_bits, wq, scale, reduce, inner / 4);
+                return;
+            }
             if (q_dtype == HIDET_QMM_I8)
                 launch(quantize4_kernel<DT, HIDET_QMM_I8, false>, dim3(cdiv(total / 4, 256)), dim3(256), 0, stream, w, amax_bits,
                        wq, scale, reduce, inner / 4, total / 4);

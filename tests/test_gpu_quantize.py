@@ -95,3 +95,38 @@ def test_benchmark_weight_shapes_bit_exact(k, n):
     assert np.all(np.abs(host(wq).astype(np.int32)).max(axis=0) == 127)
     wq2, _ = quant.symmetric_quantize(dev(-w), 'int8', dims=0)
     assert torch.equal(wq2, -wq)
+
+
+@pytest.mark.parametrize('rows,cols,qt,atype', [(1000, 4096, 'int8', 'float32'), (50, 5000, 'int8', 'float32'),
+                                               (33, 16384, 'int16', 'float32'), (9, 16388, 'int8', 'float32'),
+                                               (64, 4096, 'int8', 'float16'), (7, 1028, 'int16', 'bfloat16'),
+                                               (5, 4094, 'int8', 'float32')])
+def test_one_scale_per_row_bit_exact(rows, cols, qt, atype):
+    # embedding tables (dims=-1): rows short enough for a workgroup's registers take the one-pass kernel, longer or
+    # ragged ones the two-pass kernels; a zero row and tie values are planted
+    announce('quantize rows', rows, cols, qt, atype)
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    x[1] = 0.0
+    x[2, :8] = x[2].max() * np.array([0.5, -0.5, 1.5, -1.5, 2.5, 100.5, -100.5, 126.5], dtype=np.float32) / 127
+    if atype == 'float32':
+        t = dev(x)
+        q0, s0 = O.symmetric_quantize(x, qt, dims=-1)
+        s0b = s0.view(np.uint32)
+        view = torch.int32
+    elif atype == 'float16':
+        xh = x.astype(np.float16)
+        t = dev(xh)
+        q0, s0 = O.symmetric_quantize(xh, qt, dims=-1)
+        s0b = s0.view(np.uint16)
+        view = torch.int16
+    else:
+        xb = O.to_bf16(x)
+        t = dev(xb, torch.bfloat16)
+        q0, s0 = O.symmetric_quantize(xb, qt, dims=-1, dtype='bfloat16')
+        s0b = O.bf16_bits(s0)
+        view = torch.int16
+    wq, scale = quant.symmetric_quantize(t, qt, dims=-1)
+    assert int((host(wq) != q0).sum()) == 0
+    got = scale.view(view).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32 if view == torch.int32 else np.uint16), s0b)
