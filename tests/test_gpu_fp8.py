@@ -58,10 +58,18 @@ def test_quantize_per_tensor_every_rounding_boundary():
                           np.array([2.0 ** -10, 2.0 ** -10 * 0.99, 2.0 ** -11, 1e-12, 447.99, 440.0], dtype=np.float32)])
     pts = np.concatenate([pts, -pts]).astype(np.float32)
     pts = np.concatenate([pts, np.zeros((-pts.size) % 4, dtype=np.float32)])          # multiple of 4: the vector kernel
-    for x in (pts, pts[:-1]):                                                         # ... and the scalar one
+    big = np.tile(pts, 70000 // pts.size + 1)   # more than 65536 elements: the two-pass kernels instead of the one-launch one
+    assert big.size > 65536 and big.size % 4 == 0
+    for x in (pts, pts[:-1], big, big[:-1]):                                          # ... and the scalar ones
         codes, scale = F8.fp8_quantize_per_tensor(dev(x))
         assert scale.item() == 1.0
         assert np.array_equal(codes_of(codes), O.e4m3_encode(x))
+    for dt in (torch.float16, torch.bfloat16):                                        # narrow inputs through both paths
+        for x in (pts, big):
+            t = dev(x).to(dt)
+            codes, scale = F8.fp8_quantize_per_tensor(t)
+            assert scale.item() == 1.0
+            assert np.array_equal(codes_of(codes), O.e4m3_encode(t.float().cpu().numpy()))
 
 
 @pytest.mark.parametrize('a_shape, b_shape', [[[256, 128], [256, 128]], [[4096, 4096], [4096, 4096]], [[512, 256], [128, 256]],
