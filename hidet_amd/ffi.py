@@ -81,24 +81,34 @@ def _describe(arg) -> str:
     return str(arg)
 
 
+_FUNCS: Dict[str, object] = {}
+_Tensor = torch.Tensor
+
+
 def call(name: str, *args):
-    """Call `name` with torch tensors (passed as data pointers) and Python scalars; raise on a reported error."""
-    lib = load_library()
+    """Call `name` with torch tensors (passed as data pointers) and Python scalars; raise on a reported error.
+
+    This sits on the decode path of an eager caller (one call per linear layer and token), so it is kept short: bound
+    function objects are cached, and the error string is polled through a cached function object as well.
+    """
+    fn = _FUNCS.get(name)
+    if fn is None:
+        lib = load_library()
+        fn = _FUNCS[name] = getattr(lib, name)
+        _FUNCS.setdefault('hidet_get_last_error', lib.hidet_get_last_error)
     cargs = []
     for a in args:
-        if isinstance(a, torch.Tensor):
-            if not a.is_cuda:
+        if isinstance(a, _Tensor):
+            if not a.is_cuda:  # a host pointer must never reach a kernel
                 raise BackendException('{}: tensor argument is on {}, the kernels run on the GPU only'.format(name, a.device))
             cargs.append(a.data_ptr())
-        elif a is None:
-            cargs.append(None)
         else:
             cargs.append(a)
-    ret = getattr(lib, name)(*cargs)
-    status = get_last_error()
+    ret = fn(*cargs)
+    status = _FUNCS['hidet_get_last_error']()
     if status is not None:
         raise BackendException('Calling {} with arguments ({}) failed. error:\n{}\nFunction @ {}'.format(
-            name, ', '.join(_describe(a) for a in args), status, LIB_PATH))
+            name, ', '.join(_describe(a) for a in args), status.decode('utf-8'), LIB_PATH))
     return ret
 
 
@@ -114,7 +124,13 @@ def require_gpu(*tensors: torch.Tensor):
         dev = t.device
 
 
+_RAW_STREAM = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def current_stream(device: torch.device) -> int:
+    """Handle (hipStream_t as an integer) of torch's current stream on `device`."""
+    if _RAW_STREAM is not None:  # the same value as torch.cuda.current_stream(device).cuda_stream, without building a Stream object
+        return _RAW_STREAM(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -127,10 +143,10 @@ def workspace(device: torch.device, nbytes: int = 0) -> torch.Tensor:
     Stands in for the reference's grow-only request_hip_workspace (src/hidet/runtime/hip/context.cpp:43-57).
     One buffer per stream, because two calls that overlap in time must not share it.
     """
-    need = max(int(nbytes), int(load_library().hidet_qmm_min_workspace_bytes()))
     key = (device.index if device.index is not None else torch.cuda.current_device(), current_stream(device))
     ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < need:
+    if ws is None or ws.numel() < nbytes:
+        need = max(int(nbytes), int(load_library().hidet_qmm_min_workspace_bytes()))
         ws = torch.zeros(need, dtype=torch.uint8, device=device)
         _WORKSPACES[key] = ws
     return ws
