@@ -117,3 +117,45 @@ def test_task_descriptions():
     assert t.attrs == {'parallel_k_parts': 3} and not t.allow_prologue()
     t = SymmetricQuantizationTask(TensorSpec('w', 'float32', (32, 64)), torch.int8, dims=0)
     assert t.name == 'symmetric_quantization' and t.outputs[1].shape == (64,) and t.attrs['dims'] == [0]
+
+
+def _declared_parameter_kinds():
+    """name -> list of 'ptr' / 'i64' / 'i32' per parameter, parsed from the header's declarations."""
+    text = open(os.path.join(ROOT, 'include', 'hidet_qmm.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    out = {}
+    for m in re.finditer(r'\b(hidet_[a-z0-9_]+)\s*\(([^)]*)\)\s*;', text):
+        params = [p.strip() for p in m.group(2).split(',')]
+        if params == ['void'] or params == ['']:
+            params = []
+        kinds = []
+        for p in params:
+            if '*' in p:
+                kinds.append('ptr')
+            elif 'int64_t' in p:
+                kinds.append('i64')
+            elif re.match(r'(const\s+)?int\b', p):
+                kinds.append('i32')
+            else:
+                kinds.append(p)
+        out[m.group(1)] = kinds
+    return out
+
+
+def test_ctypes_signatures_match_the_header():
+    decl = _declared_parameter_kinds()
+    assert sorted(decl) == sorted(ffi.SIGNATURES)
+    names = {ctypes.c_void_p: 'ptr', ctypes.c_char_p: 'ptr', ctypes.c_int64: 'i64', ctypes.c_int: 'i32'}
+    for name, (_, argtypes) in ffi.SIGNATURES.items():
+        assert [names[t] for t in argtypes] == decl[name], name
+
+
+def test_header_is_plain_c():
+    import shutil
+    import subprocess
+    gcc = shutil.which('gcc')
+    if gcc is None:
+        pytest.skip('gcc not available')
+    r = subprocess.run([gcc, '-std=c99', '-Wall', '-Werror', '-fsyntax-only', '-x', 'c', os.path.join(ROOT, 'include', 'hidet_qmm.h')],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
