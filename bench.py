@@ -286,6 +286,15 @@ def main():
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ad, ws[r % RING].view(N, K), sd, cd, 1, N, K, N, 0,
                                       work, work.numel(), sptr), 48, 16)
     others['w8a16_gemv_down_proj_k11008_n4096'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * K)
+    # the same two GEMVs on weights stored K-contiguous (the [N, K] storage of torch.nn.Linear, passed as a [K, N] view):
+    # another data layout than the benchmark configuration's, so never the headline; the ring's buffers reinterpreted
+    cu = torch.empty((1, N), dtype=torch.float16, device=device)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a, ws[r % RING].view(N, K), ss[0], cu, 1, K, N, K, K,
+                                      sptr), 48, 16)
+    others['w8a16_gemv_k4096_n11008_k_contiguous_weights'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * N)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ad, ws[r % RING].view(K, N), sd, cd, 1, N, K, N, N,
+                                      sptr), 48, 16)
+    others['w8a16_gemv_down_proj_k11008_n4096_k_contiguous_weights'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * K)
     # the same GEMV kernel on a matrix five times the size (not a benchmark configuration: it shows how much of the headline
     # figure is the fixed cost of one launch and one cross-workgroup exchange)
     wl = [torch.randint(-127, 128, (8192, 28672), device=device, dtype=torch.int8) for _ in range(3)]  # 3 x 235 MB > LLC

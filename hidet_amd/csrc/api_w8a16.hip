@@ -7,6 +7,9 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
 bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda);
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+bool skinny_w8a16_nk_supported(const void *w, int64_t k, int64_t ldw);
+void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
+                            int64_t lda, int64_t ldw, hipStream_t stream);
 }
 
 using namespace qmm;
@@ -33,5 +36,21 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
         gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
         skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_symmetric_quant_matmul_f16_i8_nk(const void *a, const void *w_nk, const void *scale, void *c, int64_t m,
+                                                      int64_t k, int64_t n, int64_t lda, int64_t ldw, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
+    QMM_CHECK(lda >= k && ldw >= k, "row strides (" << lda << ", " << ldw << ") must be at least K (" << k << ")");
+    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    if (m == 0 || n == 0) return;
+    QMM_CHECK(a && w_nk && scale && c, "null tensor pointer");
+    QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
+    QMM_CHECK(skinny_w8a16_nk_supported(w_nk, k, ldw),
+              "K-contiguous weights need K and the row stride to be multiples of 16 and a 16-byte aligned pointer, got K=" << k
+                                                                                                                         << " ldw=" << ldw);
+    skinny_w8a16_nk_launch(a, w_nk, scale, c, m, k, n, lda, ldw, static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

@@ -202,3 +202,61 @@ def test_gemm_k_split_matches_unsplit_and_is_deterministic():
     ws = hidet_amd.ffi.workspace(ta.device)
     torch.cuda.synchronize()
     assert int(ws[: 64 << 10].view(torch.int32).abs().sum()) == 0
+
+
+@pytest.mark.parametrize('m,k,n', [(1, 4096, 11008), (1, 11008, 4096), (16, 4096, 4096), (3, 512, 48), (7, 144, 20), (1, 16, 2),
+                                   (20, 1024, 264), (32, 4096, 512), (2, 384, 32), (5, 1152, 8200), (4, 2176, 8192),
+                                   (9, 1040, 40)])
+def test_k_contiguous_weights_exact(m, k, n):
+    # the [K, N] weight held with strides (1, K): same operator, same results, the kernel that reduces along the
+    # contiguous axis; small integers make every product and partial sum exact.  K a multiple of 128 or not, 4 and 8
+    # waves per workgroup, waves with an empty K range, a second 16-row pass.
+    announce('w8a16 k-contiguous', m, k, n)
+    a, q, s = _int_case(m * 31 + n, m, k, n)
+    want = ((a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :])
+    want = want.astype(np.float32).astype(np.float16)
+    w_nk = quant.to_decode_layout(dev(q))
+    assert tuple(w_nk.shape) == (k, n) and w_nk.stride() == (1, k)
+    ta, ts = dev(a), dev(s)
+    # the operator: picks this kernel for a few rows and copies the weight to the row-major layout otherwise
+    assert np.array_equal(host(quant.symmetric_quant_matmul(ta, w_nk, ts)), want)
+    # the entry point itself, whatever the row count
+    c = torch.full((m, n), float('nan'), dtype=torch.float16, device='cuda')
+    hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ta, w_nk, ts, c, m, k, n, k, k,
+                       hidet_amd.ffi.current_stream(c.device))
+    assert np.array_equal(host(c), want)
+
+
+def test_k_contiguous_weights_padded_rows():
+    # rows of the stored [N, K] matrix further apart than K (a slice of a wider matrix), activations with a row stride
+    announce('w8a16 k-contiguous padded')
+    m, k, n, ldw, lda = 3, 640, 72, 1024, 768
+    a, q, s = _int_case(77, m, k, n)
+    want = ((a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :])
+    wide = torch.full((n, ldw), 99, dtype=torch.int8, device='cuda')
+    wide[:, :k] = dev(q).t()
+    abuf = torch.full((m, lda), 7.0, dtype=torch.float16, device='cuda')
+    abuf[:, :k] = dev(a)
+    got = host(quant.symmetric_quant_matmul(abuf[:, :k], wide[:, :k].t(), dev(s)))
+    assert np.array_equal(got, want.astype(np.float32).astype(np.float16))
+
+
+def test_k_contiguous_weights_parity_and_fallback():
+    announce('w8a16 k-contiguous parity')
+    a, q, s = _case(0, 1, 4096, 11008)
+    ref = clib.quant_matmul_f32acc(a, q, s)
+    w_nk = quant.to_decode_layout(dev(q))
+    got = host(quant.symmetric_quant_matmul(dev(a), w_nk, dev(s)))
+    assert O.max_rel_err(got, ref) <= 2e-3
+    # many rows, or a K that is not a multiple of 16: the weight is copied to the row-major layout and the result is the same
+    a2, q2, s2 = _int_case(5, 100, 72, 64)
+    want = ((a2.astype(np.int64) @ q2.astype(np.int64)).astype(np.float64) * s2.astype(np.float64)[None, :])
+    got2 = host(quant.symmetric_quant_matmul(dev(a2), quant.to_decode_layout(dev(q2)), dev(s2)))
+    assert np.array_equal(got2, want.astype(np.float32).astype(np.float16))
+    # the C entry point refuses what it cannot take
+    from hidet_amd import ffi
+    bad = torch.zeros(8, 24, device='cuda', dtype=torch.int8)
+    with pytest.raises(hidet_amd.BackendException):
+        ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', torch.zeros(1, 24, device='cuda', dtype=torch.float16), bad,
+                 torch.zeros(8, device='cuda', dtype=torch.float16), torch.zeros(1, 8, device='cuda', dtype=torch.float16),
+                 1, 24, 8, 24, 24, ffi.current_stream(bad.device))
