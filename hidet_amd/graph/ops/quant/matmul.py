@@ -4,6 +4,8 @@ from typing import List
 
 import torch
 
+from torch.utils.weak import WeakTensorKeyDictionary
+
 from hidet_amd import ffi, option
 from hidet_amd.graph.operator import Operator, Task, TensorSpec, input_like
 
@@ -62,6 +64,23 @@ def to_decode_layout(wq: torch.Tensor) -> torch.Tensor:
     return wq.t().contiguous().t()
 
 
+_ROW_MAJOR_COPIES = WeakTensorKeyDictionary()  # K-contiguous weight tensor (by identity) -> its row-major copy
+
+
+def _row_major(weight: torch.Tensor) -> torch.Tensor:
+    """`weight` as the row-major [K, N] tensor the GEMM and the N-contiguous GEMV read.  The copy of a K-contiguous weight
+    (45 MB for a 4096 x 11008 layer) is made once per tensor object and lives as long as that object does; a weight that
+    is modified in place afterwards must be passed as a new tensor."""
+    if weight.is_contiguous():
+        return weight
+    if weight.dim() == 2 and weight.stride(0) == 1:
+        copy = _ROW_MAJOR_COPIES.get(weight)
+        if copy is None or copy.device != weight.device:
+            copy = _ROW_MAJOR_COPIES[weight] = weight.contiguous()
+        return copy
+    return weight.contiguous()
+
+
 def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parallel_k_parts: int = 0) -> torch.Tensor:
     """c[..., M, N] on the GPU.  Leading axes of `a` are folded into M: the weight is 2-D, so broadcasting
     over them is the same as one tall matmul."""
@@ -82,7 +101,7 @@ def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parall
         ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a2, weight, scale, c, m, k, n, lda, weight.stride(1),
                  ffi.current_stream(a.device))
         return c.reshape(tuple(a.shape[:-1]) + (n,))
-    weight = weight.contiguous()
+    weight = _row_major(weight)
     ws = ffi.workspace(a.device)
     ffi.call('hidet_symmetric_quant_matmul_f16_i8', a2, weight, scale, c, m, k, n, lda, int(parallel_k_parts), ws,
              ws.numel(), ffi.current_stream(a.device))

@@ -37,6 +37,7 @@ class PassContext:
             'precision': None,            # target float dtype of the model: None, 'float16', 'bfloat16', 'float32'
             'quantize_patterns': [],      # selective quantization rules, applied in order
             'quantized_weights': None,    # optional QuantizedWeightStore: reuse persisted (wq, scale) instead of quantizing
+            'decode_layout': False,       # keep the int8 codes of fused linears K-contiguous (see set_decode_layout)
             'verbose': False,
         }
         self.rewrites: List[Tuple[str, int]] = []  # (rule name, sub-graphs rewritten), filled by the passes
@@ -87,6 +88,16 @@ class PassContext:
         """Weights quantized earlier (see hidet_amd.graph.frontend.torch.QuantizedWeightStore): the linear and embedding
         rules take (wq, scale) from the store when it has the parameter's name instead of quantizing again."""
         self.configs['quantized_weights'] = store
+        return self
+
+    def set_decode_layout(self, enable: bool = True) -> 'PassContext':
+        """Keep the int8 codes of every fused linear layer K-contiguous (the storage order of `nn.Linear.weight`).
+
+        Calls with a few activation rows (token-by-token decoding) then run the GEMV that reduces along the contiguous
+        axis; a call with more rows makes a row-major copy of the codes the first time and keeps it, so a model that
+        does both holds the int8 weights twice. No counterpart in the reference, whose quantized operator reads
+        row-major `[K, N]` codes only (python/hidet/graph/ops/quant/matmul.py:24-74)."""
+        self.configs['decode_layout'] = bool(enable)
         return self
 
     def set_verbose(self, verbose: bool = True) -> 'PassContext':

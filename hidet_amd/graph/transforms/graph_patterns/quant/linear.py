@@ -184,7 +184,11 @@ class SymmetricQuantizeMatmulFused(SubgraphRewriteRule):
             if x_dtype != torch.float16 or scale.dtype != torch.float16:
                 continue
             with gm.graph.inserting_before(node):
-                out = gm.graph.call_function(quant.symmetric_quant_matmul, (x, w_dequant.args[0], w_dequant.args[1]))
+                wq_node = w_dequant.args[0]
+                if ctx.configs.get('decode_layout'):
+                    # same [K, N] operand, stored K-contiguous; the row-major constant loses its last user below
+                    wq_node = gm.graph.get_attr(add_constant(gm, wq_node.target + '_kc', quant.to_decode_layout(wq)))
+                out = gm.graph.call_function(quant.symmetric_quant_matmul, (x, wq_node, w_dequant.args[1]))
             out.meta = dict(node.meta)
             node.replace_all_uses_with(out)
             gm.graph.erase_node(node)

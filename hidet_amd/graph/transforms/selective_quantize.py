@@ -17,7 +17,19 @@ class SelectiveQuantizePass(GraphPass):
                 gm.graph.eliminate_dead_code()
                 gm.graph.lint()
                 gm.recompile()
+        _release_unused_constants(gm)
         return gm
+
+
+def _release_unused_constants(gm: fx.GraphModule):
+    """Drop what the rewritten graph no longer reads: sub-modules that are not called any more (the float weights of
+    quantized linear layers and embeddings) and buffers of the root module that no `get_attr` node names (codes that a
+    later rule replaced by another layout)."""
+    gm.delete_all_unused_submodules()
+    used = {str(n.target) for n in gm.graph.nodes if n.op == 'get_attr'}
+    for name in [n for n, _ in gm.named_buffers(recurse=False)]:
+        if name not in used:
+            delattr(gm, name)
 
 
 def selective_quantize_pass() -> GraphPass:

@@ -120,3 +120,33 @@ def test_ahead_of_time_rewrite_and_persisted_weights(tmp_path):
         gm2 = quantize_module(blank, ctx)
     with torch.no_grad():
         assert torch.equal(gm2(x.half()), got)
+
+
+def test_decode_layout_runs_decode_and_prefill_calls():
+    announce('graph rewrite: decode layout')
+    torch.manual_seed(3)
+
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up, self.down = torch.nn.Linear(512, 1024), torch.nn.Linear(1024, 512, bias=False)
+
+        def forward(self, x):
+            return self.down(F.gelu(self.up(x)))
+
+    model = Mlp().cuda().eval()
+    with PassContext() as ctx:
+        ctx.set_precision('int8')
+        plain = quantize_module(model, ctx)
+    with PassContext() as ctx:
+        ctx.set_precision('int8').set_decode_layout()
+        gm = quantize_module(model, ctx)
+    assert gm.up_weight_wq_kc.stride() == (1, 512) and torch.equal(gm.up_weight_wq_kc, plain.up_weight_wq)
+    for rows in (1, 3, 40, 16, 1):  # decode-sized calls, a prefill-sized one (row-major copy made once), decode again
+        x = torch.randn(rows, 512, device='cuda', dtype=torch.float16)
+        with torch.no_grad():
+            got, want = gm(x), plain(x)
+        assert got.shape == want.shape
+        assert O.max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) < 2e-3
+    from hidet_amd.graph.ops.quant import matmul as qmm
+    assert qmm._ROW_MAJOR_COPIES.get(gm.up_weight_wq_kc) is not None

@@ -107,6 +107,32 @@ def test_linear_modules_become_fused_operator(cpu_ops):
     assert O.max_rel_err(got.float().numpy(), want.detach().numpy()) < 3e-2
 
 
+def test_decode_layout_keeps_codes_k_contiguous_and_releases_the_rest(cpu_ops):
+    torch.manual_seed(2)
+    model = Mlp().eval()
+    x = torch.randn(2, 32)
+    want = model(x)
+    with PassContext() as ctx:
+        ctx.set_precision('int8').set_decode_layout()
+        assert ctx.configs['decode_layout'] is True
+        gm = quantize_module(model, ctx)
+    consts = {n: b for n, b in gm.named_buffers()}
+    # one int8 constant per layer, [K, N] with K contiguous; the row-major codes and the float modules are gone
+    assert sorted(consts) == ['down_bias', 'down_weight_scale', 'down_weight_wq_kc', 'up_bias', 'up_weight_scale', 'up_weight_wq_kc']
+    up = consts['up_weight_wq_kc']
+    assert tuple(up.shape) == (32, 64) and up.stride() == (1, 32) and up.dtype == torch.int8
+    assert not hasattr(gm, 'up') and not hasattr(gm, 'down')
+    q, _ = O.symmetric_quantize(model.up.weight.detach().half().t().contiguous().numpy(), 'int8', dims=0)
+    assert np.array_equal(up.numpy(), q)
+    got = gm(x.half())
+    assert O.max_rel_err(got.float().numpy(), want.detach().numpy()) < 3e-2
+    # without the option nothing changes in the constants' layout, and unused float modules are released all the same
+    with PassContext() as ctx:
+        ctx.set_precision('int8')
+        gm2 = quantize_module(Mlp().eval(), ctx)
+    assert gm2.up_weight_wq.is_contiguous() and not hasattr(gm2, 'up')
+
+
 def test_functional_linear_matmul_right_and_left(cpu_ops):
     class M(torch.nn.Module):
         def __init__(self):
