@@ -278,6 +278,9 @@ def main():
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', a16, w16[r % 32], s16, c16, 16, 4096, 4096, 4096, 0,
                                       work, work.numel(), sptr), 96, 32)
     others['w8a16_m16_k4096_n4096'] = hbm_entry(us, 4096 * 4096 + 2 * 4096 + 2 * 16 * 4096 * 2)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a16, w16[r % 32], s16, c16, 16, 4096, 4096, 4096, 4096,
+                                      sptr), 96, 32)  # the same buffers read as [N, K] storage
+    others['w8a16_m16_k4096_n4096_k_contiguous_weights'] = hbm_entry(us, 4096 * 4096 + 2 * 4096 + 2 * 16 * 4096 * 2)
     del w16
     # W8A16 decode GEMV, down-proj shape [1, 11008] x [11008, 4096]: the ring's buffers reinterpreted as [11008, 4096]
     ad = torch.randn((1, N), generator=g, device=device, dtype=torch.float32).to(torch.float16)

@@ -20,13 +20,21 @@ namespace qmm {
 namespace {
 
 
-template <bool ALIGNED_A, bool FULL, int WAVES>
+template <bool ALIGNED_A, bool FULL, int WAVES, bool STAGE = false>
 __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Float16 *__restrict__ a, int64_t lda,
                                                               const int8_t *__restrict__ w, int64_t ldw,
                                                               const _Float16 *__restrict__ scale, _Float16 *__restrict__ c,
                                                               int m, int k, int n) {
     __shared__ float red[WAVES][16][17];
     constexpr int kNkDepth = FULL ? 8 : 4;  // 128-deep steps whose loads are issued together
+    // STAGE (FULL with aligned activations, more than two rows): a wave fetches its 16 x 128 activation block of a step
+    // with four fully coalesced loads (4 rows x 256 bytes each) and turns it into MFMA fragments through a private LDS
+    // tile of 16 rows x (256 + 16) bytes, two slots.  Fetching the fragments straight from memory touches every cache
+    // line of the block four times, and made 16 rows cost 8 us more than one; with one or two rows the direct fetch
+    // is a broadcast and a little faster.  No barrier: the LDS operations of one wave execute in order.
+    static_assert(!STAGE || (FULL && ALIGNED_A), "staging needs the condition-free loop and 16-byte loads");
+    constexpr bool kStage = STAGE;
+    __shared__ uint4 stage[kStage ? WAVES : 1][2][16 * 17];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 4, ls = lane & 15;
@@ -50,6 +58,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
     for (int s0 = s_begin; s0 < s_end; s0 += kNkDepth) {
         uint4 wv[kNkDepth][2];
         half8_t xa[kNkDepth][4];
+        uint4 ax[kStage ? kNkDepth : 1][4];
 #pragma unroll
         for (int d = 0; d < kNkDepth; ++d) {
             if (FULL) {
@@ -72,7 +81,10 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
             for (int j = 0; j < 4; ++j) {
                 if (FULL) {
                     const int st = min(s0 + d, s_end - 1);
-                    if (ALIGNED_A) {
+                    if (kStage) {  // load j: rows 4j .. 4j+3, 16 lanes x 16 bytes per row
+                        const int r = min(4 * j + kg, m - 1);
+                        ax[d][j] = *reinterpret_cast<const uint4 *>(a + int64_t(r) * lda + int64_t(st) * 128 + 8 * ls);
+                    } else if (ALIGNED_A) {
                         xa[d][j] = *reinterpret_cast<const half8_t *>(ap + int64_t(st) * 128 + 8 * j);
                     } else {
 #pragma unroll
@@ -95,6 +107,13 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
 #pragma unroll
         for (int d = 0; d < kNkDepth; ++d) {
             if (FULL && s0 + d >= s_end) break;  // wave-uniform
+            if (kStage) {
+                uint4 *tile = stage[wave][d & 1];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) tile[(4 * j + kg) * 17 + ls] = ax[d][j];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xa[d][j] = __builtin_bit_cast(half8_t, tile[ls * 17 + 4 * kg + j]);
+            }
             const uint32_t raw[8] = {wv[d][0].x, wv[d][0].y, wv[d][0].z, wv[d][0].w, wv[d][1].x, wv[d][1].y, wv[d][1].z, wv[d][1].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -127,6 +146,105 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
     }
 }
 
+// More than a few activation rows: the kernel above re-reads the activation rows once per 16 output columns, which at 16
+// rows is twice the weight bytes.  Here a wave keeps one activation fragment for CG column groups (16 CG columns per
+// workgroup), so that traffic drops by CG; the workgroup's waves split K as before.  K a multiple of 128, aligned
+// activations; the loop has no conditions (clamped rows, see above).
+template <int CG, int WAVES, int DEPTH>
+__global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_wide_kernel(const _Float16 *__restrict__ a, int64_t lda,
+                                                                          const int8_t *__restrict__ w, int64_t ldw,
+                                                                          const _Float16 *__restrict__ scale,
+                                                                          _Float16 *__restrict__ c, int m, int k, int n) {
+    __shared__ float red[WAVES][CG][16][17];
+    __shared__ uint4 stage[WAVES][2][16 * 17];  // per wave: activation block of a step, see the kernel above
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 4, ls = lane & 15;
+    const int n0 = blockIdx.x * (16 * CG);
+
+    const int steps = k >> 7;
+    const int steps_per_wave = (steps + WAVES - 1) / WAVES;
+    const int s_begin = wave * steps_per_wave, s_end = min(steps, s_begin + steps_per_wave);
+
+    float4_t acc[CG], xsum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < CG; ++g) acc[g] = float4_t{0.f, 0.f, 0.f, 0.f};
+    half8_t ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = _Float16(1.0f);
+    const int8_t *wp[CG];
+#pragma unroll
+    for (int g = 0; g < CG; ++g) wp[g] = w + int64_t(min(n0 + 16 * g + ls, n - 1)) * ldw + 32 * kg;
+
+    for (int s0 = s_begin; s0 < s_end; s0 += DEPTH) {
+        uint4 wv[DEPTH][CG][2];
+        half8_t xa[DEPTH][4];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int st = min(s0 + d, s_end - 1);  // a step past the wave's range re-reads its last one; not used
+#pragma unroll
+            for (int g = 0; g < CG; ++g) {
+                wv[d][g][0] = *reinterpret_cast<const uint4 *>(wp[g] + int64_t(st) * 128);
+                wv[d][g][1] = *reinterpret_cast<const uint4 *>(wp[g] + int64_t(st) * 128 + 16);
+            }
+        }
+        uint4 ax[DEPTH][4];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int st = min(s0 + d, s_end - 1);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = min(4 * j + kg, m - 1);
+                ax[d][j] = *reinterpret_cast<const uint4 *>(a + int64_t(r) * lda + int64_t(st) * 128 + 8 * ls);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (s0 + d >= s_end) break;  // wave-uniform
+            uint4 *tile = stage[wave][d & 1];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tile[(4 * j + kg) * 17 + ls] = ax[d][j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xa[d][j] = __builtin_bit_cast(half8_t, tile[ls * 17 + 4 * kg + j]);
+#pragma unroll
+            for (int g = 0; g < CG; ++g) {
+                const uint32_t raw[8] = {wv[d][g][0].x, wv[d][g][0].y, wv[d][g][0].z, wv[d][g][0].w,
+                                         wv[d][g][1].x, wv[d][g][1].y, wv[d][g][1].z, wv[d][g][1].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    constexpr uint32_t kLo = 0x0c010c00u, kHi = 0x0c030c02u;
+                    union {
+                        uint32_t u[4];
+                        half8_t h8;
+                    } b;
+                    b.u[0] = __builtin_amdgcn_perm(raw[2 * j], raw[2 * j], kLo) ^ 0x64806480u;
+                    b.u[1] = __builtin_amdgcn_perm(raw[2 * j], raw[2 * j], kHi) ^ 0x64806480u;
+                    b.u[2] = __builtin_amdgcn_perm(raw[2 * j + 1], raw[2 * j + 1], kLo) ^ 0x64806480u;
+                    b.u[3] = __builtin_amdgcn_perm(raw[2 * j + 1], raw[2 * j + 1], kHi) ^ 0x64806480u;
+                    acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[d][j], b.h8, acc[g], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[d][j], ones, xsum, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < CG; ++g)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][g][4 * kg + v][ls] = acc[g][v] - 1152.0f * xsum[v];
+    __syncthreads();
+    for (int o = tid; o < CG * 256; o += 64 * WAVES) {
+        const int g = o >> 8, row = (o >> 4) & 15, cn = o & 15;
+        const int col = n0 + 16 * g + cn;
+        if (row < m && col < n) {
+            float v = 0.f;
+#pragma unroll
+            for (int p = 0; p < WAVES; ++p) v += red[p][g][row][cn];
+            c[int64_t(row) * n + col] = _Float16(v * float(scale[col]));
+        }
+    }
+}
+
 }  // namespace
 
 bool skinny_w8a16_nk_supported(const void *w, int64_t k, int64_t ldw) {
@@ -148,9 +266,18 @@ void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, voi
                    cp, mt, int(k), int(n));
         };
         const bool full = k % 128 == 0;
+        // more than 8 rows, a wide matrix and a long K: 32 columns per workgroup, the activation rows are read half as often
+        if (full && aligned_a && mt > 8 && cdiv(n, 32) >= 256 && k >= 8192) {
+            launch(skinny_w8a16_nk_wide_kernel<2, 8, 4>, dim3(uint32_t(cdiv(n, 32))), dim3(512), 0, stream, ap, lda,
+                   static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale), cp, mt, int(k), int(n));
+            continue;
+        }
         // few column tiles: eight waves per workgroup keep enough loads in flight on each compute unit
         const bool eight = full && cdiv(n, 16) < 512 && k >= 8 * 128;
-        if (eight) aligned_a ? go(skinny_w8a16_nk_kernel<true, true, 8>, 8) : go(skinny_w8a16_nk_kernel<false, true, 8>, 8);
+        const bool stage = full && aligned_a && mt > 2;
+        if (eight && stage) go(skinny_w8a16_nk_kernel<true, true, 8, true>, 8);
+        else if (eight) aligned_a ? go(skinny_w8a16_nk_kernel<true, true, 8>, 8) : go(skinny_w8a16_nk_kernel<false, true, 8>, 8);
+        else if (stage) go(skinny_w8a16_nk_kernel<true, true, 4, true>, 4);
         else if (aligned_a) full ? go(skinny_w8a16_nk_kernel<true, true, 4>, 4) : go(skinny_w8a16_nk_kernel<true, false, 4>, 4);
         else full ? go(skinny_w8a16_nk_kernel<false, true, 4>, 4) : go(skinny_w8a16_nk_kernel<false, false, 4>, 4);
     }

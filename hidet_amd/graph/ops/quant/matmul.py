@@ -40,24 +40,16 @@ class SymmetricQuantizedMatmulTask(Task):
                          outputs=[TensorSpec('c', 'float16', c_shape)], attrs={})
 
 
-def _nk_max_rows(n: int) -> int:
-    """Most activation rows for which K-contiguous weights go to the kernel that reduces along the contiguous axis.
-
-    That kernel re-reads the activation rows once per 16 output columns, so its time grows with the row count, while the
-    kernel for N-contiguous weights costs the same for 1 to 16 rows: measured at K = 4096, N = 11008 the former wins up to
-    4 rows (11.7 / 12.5 / 13.1 us against 14.1 us) and loses from 8 (15.7 us); with fewer than 512 column groups (N < 8192)
-    the N-contiguous kernel cannot fill the chip and the K-contiguous one wins for every row count of a pass.
-    """
-    return 16 if (n + 15) // 16 < 512 else 4
+_NK_MAX_ROWS = 16  # one pass of the K-contiguous kernel; more rows are served better by the MFMA GEMM on row-major codes
 
 
 def to_decode_layout(wq: torch.Tensor) -> torch.Tensor:
     """The same [K, N] int8 weight, stored K-contiguous (a view with strides (1, K) of a fresh [N, K] tensor).
 
-    `symmetric_quant_matmul` on such a weight with a few activation rows (see `_nk_max_rows`) runs the kernel that
+    `symmetric_quant_matmul` on such a weight with up to 16 activation rows runs the kernel that
     reduces along the contiguous axis (no exchange between workgroups); it is what `nn.Linear` stores, so `linear.weight`
-    quantized with `dims=1` and viewed with `.t()` is already in this layout.  Calls with more rows copy the weight to the
-    row-major layout first, as for any non-contiguous operand: keep a row-major copy for prefill.
+    quantized with `dims=1` and viewed with `.t()` is already in this layout.  A call with more rows makes a row-major copy
+    of the weight the first time and keeps it for as long as the weight tensor lives.
     """
     if wq.dim() != 2:
         raise ValueError('expected a 2-D weight, got shape {}'.format(list(wq.shape)))
@@ -96,7 +88,7 @@ def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parall
     # A [K, N] weight held K-contiguous (strides (1, ldw): `wq_nk.t()` of an [N, K] tensor, see `to_decode_layout`) goes to the
     # kernel that reduces along the contiguous axis when the call is a decode-sized one; otherwise it is copied to the
     # row-major layout the other kernels read, as any non-contiguous operand is.
-    if (m <= _nk_max_rows(n) and k > 1 and n > 1 and weight.stride(0) == 1 and weight.stride(1) >= k and weight.stride(1) % 16 == 0
+    if (m <= _NK_MAX_ROWS and k > 1 and n > 1 and weight.stride(0) == 1 and weight.stride(1) >= k and weight.stride(1) % 16 == 0
             and k % 16 == 0 and weight.data_ptr() % 16 == 0):
         ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a2, weight, scale, c, m, k, n, lda, weight.stride(1),
                  ffi.current_stream(a.device))
