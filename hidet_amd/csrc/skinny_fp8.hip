@@ -98,6 +98,79 @@ __global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restri
     }
 }
 
+// 3 to 16 rows, K a multiple of 128, aligned activations.  Fetching the activation operand straight from memory (lane =
+// 16 bytes at a 32-byte stride of one of 16 rows) touches every cache line of a step's 16 x 128-byte block twice and once
+// per row, and the time grew with M (8192 x 8192: 13.3 us for one row, 19.6 us for 16).  Here a wave fetches the block
+// with two fully coalesced loads (8 rows x 128 bytes each) and reads its operand back from a private LDS tile of
+// 16 rows x (128 + 16) bytes, two slots; no barrier, one wave's LDS operations execute in order.  The loop has no
+// conditions: lanes of rows >= M and columns >= N read a clamped row and their results are dropped.
+template <int OUT>
+__global__ __launch_bounds__(256) void skinny_fp8_staged_kernel(const uint8_t *__restrict__ a, int64_t lda,
+                                                                const uint8_t *__restrict__ b, int64_t ldb,
+                                                                void *__restrict__ c, int m, int n, int k,
+                                                                const float *__restrict__ scale_a,
+                                                                const float *__restrict__ scale_b) {
+    __shared__ float red[kWaves][16][17];
+    __shared__ uint4 stage[kWaves][2][16 * 9];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 4, ls = lane & 15;
+    const int n0 = blockIdx.x * 16;
+
+    const int steps = k >> 7;
+    const int steps_per_wave = (steps + kWaves - 1) / kWaves;
+    const int s_begin = wave * steps_per_wave, s_end = min(steps, s_begin + steps_per_wave);
+
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const uint8_t *bp = b + int64_t(min(n0 + ls, n - 1)) * ldb + 32 * kg;
+    const uint8_t *ap0 = a + int64_t(min(lane >> 3, m - 1)) * lda + 16 * (lane & 7);
+    const uint8_t *ap1 = a + int64_t(min(8 + (lane >> 3), m - 1)) * lda + 16 * (lane & 7);
+
+    for (int s0 = s_begin; s0 < s_end; s0 += kDepth) {
+        uint4 wv[kDepth][2], ax[kDepth][2];
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            const int st = min(s0 + d, s_end - 1);  // a step past the wave's range re-reads its last one; not used
+            wv[d][0] = *reinterpret_cast<const uint4 *>(bp + int64_t(st) * 128);
+            wv[d][1] = *reinterpret_cast<const uint4 *>(bp + int64_t(st) * 128 + 16);
+        }
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            const int st = min(s0 + d, s_end - 1);
+            ax[d][0] = *reinterpret_cast<const uint4 *>(ap0 + int64_t(st) * 128);
+            ax[d][1] = *reinterpret_cast<const uint4 *>(ap1 + int64_t(st) * 128);
+        }
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            if (s0 + d >= s_end) break;  // wave-uniform
+            uint4 *tile = stage[wave][d & 1];
+            tile[(lane >> 3) * 9 + (lane & 7)] = ax[d][0];
+            tile[(8 + (lane >> 3)) * 9 + (lane & 7)] = ax[d][1];
+            const uint4 x0 = tile[ls * 9 + 2 * kg], x1 = tile[ls * 9 + 2 * kg + 1];
+            int8v_t rv, cv;
+            rv[0] = int(x0.x); rv[1] = int(x0.y); rv[2] = int(x0.z); rv[3] = int(x0.w);
+            rv[4] = int(x1.x); rv[5] = int(x1.y); rv[6] = int(x1.z); rv[7] = int(x1.w);
+            cv[0] = int(wv[d][0].x); cv[1] = int(wv[d][0].y); cv[2] = int(wv[d][0].z); cv[3] = int(wv[d][0].w);
+            cv[4] = int(wv[d][1].x); cv[5] = int(wv[d][1].y); cv[6] = int(wv[d][1].z); cv[7] = int(wv[d][1].w);
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][4 * kg + v][ls] = acc[v];
+    __syncthreads();
+    const int row = tid >> 4, cn = tid & 15;
+    if (row < m && n0 + cn < n) {
+        float v = red[0][row][cn] + red[1][row][cn] + red[2][row][cn] + red[3][row][cn];
+        if (scale_a != nullptr) v *= *scale_a;
+        if (scale_b != nullptr) v *= *scale_b;
+        const int64_t o = int64_t(row) * n + n0 + cn;
+        if (OUT == HIDET_QMM_F32) static_cast<float *>(c)[o] = v;
+        else if (OUT == HIDET_QMM_BF16) static_cast<uint16_t *>(c)[o] = f32_to_bf16_bits(v);
+        else if (OUT == HIDET_QMM_F16) static_cast<uint16_t *>(c)[o] = f32_to_f16_bits(v);
+        else static_cast<uint8_t *>(c)[o] = f32_to_e4m3(v);
+    }
+}
+
 }  // namespace
 
 bool skinny_fp8_supported(const void *b, int64_t k, int64_t ldb) { return (ldb % 16 == 0) && (k % 16 == 0) && aligned(b, 16) && k > 0; }
@@ -109,8 +182,10 @@ void skinny_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t
     const bool aligned_a = (lda % 16 == 0) && aligned(a, 16);
     const dim3 grid(uint32_t(cdiv(n, 16)));
     auto go = [&](auto kern) { launch(kern, grid, dim3(256), 0, stream, ap, lda, bp, ldb, c, int(m), int(n), int(k), sa, sb); };
+    const bool staged = aligned_a && k % 128 == 0;
 #define QMM_FP8_SKINNY(OUT)                                   \
-    if (aligned_a) go(skinny_fp8_kernel<OUT, true>);          \
+    if (staged) go(skinny_fp8_staged_kernel<OUT>);            \
+    else if (aligned_a) go(skinny_fp8_kernel<OUT, true>);     \
     else go(skinny_fp8_kernel<OUT, false>);
     switch (out_dtype) {
         case HIDET_QMM_F32: QMM_FP8_SKINNY(HIDET_QMM_F32) break;
