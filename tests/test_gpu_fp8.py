@@ -167,6 +167,24 @@ def test_k_split_is_deterministic_and_optional():
     assert O.max_rel_err(first, ref) <= 1e-5
 
 
+@pytest.mark.parametrize('m,k,n', [(1, 128, 16), (3, 384, 40), (7, 1152, 72), (16, 8192, 8192), (2, 4096, 4096), (16, 2048, 8200),
+                                   (5, 1040, 48), (9, 11008, 520), (13, 1024, 24)])
+def test_skinny_exact_on_small_integers(m, k, n):
+    # 1..16 rows: integer operands make every product and partial sum exact, so the result must be the integer
+    # product whichever kernel runs (K a multiple of 128 or not, 4 or 8 waves, waves with an empty K range,
+    # columns that do not fill the last workgroup), also for a row stride larger than K
+    announce('fp8 skinny exact', m, k, n)
+    rng = np.random.default_rng(m * 1000 + n)
+    ai, bi = rng.integers(-4, 5, (m, k)), rng.integers(-4, 5, (n, k))
+    want = ai.astype(np.int64) @ bi.astype(np.int64).T
+    ta, tb = f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32)))
+    assert np.array_equal(host(F8.matmul_f8(ta, tb, output_dtype='float32')).astype(np.int64), want)
+    wide = torch.full((m, k + 256), 0x38, dtype=torch.uint8, device='cuda')  # 1.0 outside the operand
+    wide[:, 128:128 + k] = ta.view(torch.uint8)
+    got = F8.matmul_f8(wide[:, 128:128 + k].view(torch.float8_e4m3fn), tb, output_dtype='float32')
+    assert np.array_equal(host(got).astype(np.int64), want)
+
+
 def test_batched_and_strided_operands():
     announce('fp8 batched')
     rng = np.random.default_rng(5)
