@@ -5,11 +5,11 @@
 // 2j+1), scales are [K / group, N] in the activation dtype (bfloat16 or float16).  Same structure as the
 // int8 kernel: lane (g, cl) loads rows 8g .. 8g+7 of a 32-row k-step, 8 bytes = 16 columns per row, so a
 // load instruction covers four 128-byte row segments and a wave covers 256 columns.  The nibbles are
-// split into even and odd columns with two masks, byte-gathered pairwise across two rows with
-// v_perm_b32, and one v_xor_b32 produces two bfloat16 (0x4300 | (nibble ^ 8) == 136 + q) or float16
-// (0x6400 | (nibble ^ 8) == 1032 + q) values: the B operand of a 16x16x32 MFMA.  The constant is removed
-// per group with one extra MFMA against ones; at every group boundary the fp32 accumulators are scaled
-// into the running totals.
+// byte-gathered pairwise across two rows with v_perm_b32 (one byte = an even and an odd column), and a
+// mask-and-xor (one three-input bit operation; plus a shift for the odd column) produces two bfloat16
+// (0x4300 | (nibble ^ 8) == 136 + q) or float16 (0x6400 | (nibble ^ 8) == 1032 + q) values: the B operand
+// of a 16x16x32 MFMA.  The constant is removed per group with one extra MFMA against ones; at every group
+// boundary the fp32 accumulators are scaled into the running totals.
 #include "skinny_common.h"
 
 namespace qmm {
@@ -38,7 +38,7 @@ struct W4Traits<HIDET_QMM_F16> {
     static __device__ __forceinline__ float to_f32(uint16_t b) { return f16_bits_to_f32(b); }
 };
 
-template <int DT, int DEPTH, bool ALIGNED_A>
+template <int DT, int DEPTH, bool ALIGNED_A, bool FULL = false>
 __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,
                                                            const uint8_t *__restrict__ w,
                                                            const uint16_t *__restrict__ scales, uint16_t *__restrict__ c,
@@ -73,8 +73,10 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
     const uint32_t one2 = uint32_t(T::kOne) | (uint32_t(T::kOne) << 16);
     const uint4 ones = uint4{one2, one2, one2, one2};
 
+    // FULL: every column exists, every wave's K range is a whole number of iterations and the activations allow 16-byte
+    // loads, so the loop has no per-lane conditions; lanes of rows >= M read the last row and their results are dropped
     const uint8_t *wp = w + (col0 >> 1);
-    const uint16_t *ap = a + int64_t(cl) * lda;
+    const uint16_t *ap = a + int64_t(FULL ? min(cl, m - 1) : cl) * lda;
     uint4 sc_raw[2] = {uint4{0u, 0u, 0u, 0u}, uint4{0u, 0u, 0u, 0u}};  // 16 scales of the current group
 
     for (int kk = k_begin; kk < k_end; kk += 32 * DEPTH) {
@@ -85,12 +87,20 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int row = kk + 32 * d + 8 * g + j;
+                if (FULL) {
+                    raw[d][j] = *reinterpret_cast<const uint2 *>(wp + int64_t(row) * row_bytes);
+                    continue;
+                }
                 raw[d][j] = uint2{0x88888888u, 0x88888888u};  // nibble 8 ^ 8 == code 0
                 if (col_ok && row < k_end) raw[d][j] = *reinterpret_cast<const uint2 *>(wp + int64_t(row) * row_bytes);
             }
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int kx = kk + 32 * d + 8 * g;
+            if (FULL) {
+                xa[d] = *reinterpret_cast<const uint4 *>(ap + kx);
+                continue;
+            }
             xa[d] = uint4{0u, 0u, 0u, 0u};
             if (cl < m) {
                 if (ALIGNED_A) {
@@ -107,39 +117,36 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             const int ks = kk + 32 * d;
-            if (ks < k_end) {  // uniform across the wave
+            if (FULL || ks < k_end) {  // uniform across the wave
                 if (ks % group == 0 || ks == k_begin) {
-                    if (col_ok) {
+                    if (FULL || col_ok) {
                         const uint16_t *sp = scales + int64_t(ks / group) * n + col0;
                         sc_raw[0] = *reinterpret_cast<const uint4 *>(sp);
                         sc_raw[1] = *reinterpret_cast<const uint4 *>(sp + 8);
                     }
                 }
-                // split the nibbles of one dword column at a time: ev[j] holds columns 8h + {0,2,4,6} of row j
-                // in its 4 bytes, od[j] the odd ones
+                // byte b of dword h of rows 2p and 2p+1 goes to bits 0-7 and 16-23 of one register (v_perm_b32); its low
+                // nibbles are column 8h + 2b of both rows, its high nibbles column 8h + 2b + 1: mask-and-xor (one
+                // three-input bit operation) gives the two 16-bit floats bias + q, for the odd column after a shift
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    uint32_t ev[8], od[8];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const uint32_t r = h ? raw[d][j].y : raw[d][j].x;
-                        ev[j] = r & 0x0F0F0F0Fu;
-                        od[j] = (r >> 4) & 0x0F0F0F0Fu;
-                    }
-#pragma unroll
-                    for (int nb = 0; nb < 8; ++nb) {
+                    for (int byte = 0; byte < 4; ++byte) {
                         constexpr uint32_t kZero = 0x0c;
-                        const int t = 8 * h + nb, byte = nb >> 1;
                         const uint32_t sel = (kZero << 24) | (uint32_t(4 + byte) << 16) | (kZero << 8) | uint32_t(byte);
-                        uint4 b;
-                        uint32_t *bp = reinterpret_cast<uint32_t *>(&b);
+                        uint4 be, bo;
+                        uint32_t *bep = reinterpret_cast<uint32_t *>(&be), *bop = reinterpret_cast<uint32_t *>(&bo);
 #pragma unroll
                         for (int p = 0; p < 4; ++p) {
-                            const uint32_t lo = (nb & 1) ? od[2 * p] : ev[2 * p];
-                            const uint32_t hi = (nb & 1) ? od[2 * p + 1] : ev[2 * p + 1];
-                            bp[p] = __builtin_amdgcn_perm(hi, lo, sel) ^ T::kMagic;
+                            const uint32_t lo = h ? raw[d][2 * p].y : raw[d][2 * p].x;
+                            const uint32_t hi = h ? raw[d][2 * p + 1].y : raw[d][2 * p + 1].x;
+                            const uint32_t x = __builtin_amdgcn_perm(hi, lo, sel);
+                            bep[p] = (x & 0x000F000Fu) ^ T::kMagic;
+                            bop[p] = ((x >> 4) & 0x000F000Fu) ^ T::kMagic;
                         }
-                        acc[t] = T::mfma(xa[d], b, acc[t]);
+                        const int t = 8 * h + 2 * byte;
+                        acc[t] = T::mfma(xa[d], be, acc[t]);
+                        acc[t + 1] = T::mfma(xa[d], bo, acc[t + 1]);
                     }
                 }
                 xsum = T::mfma(xa[d], ones, xsum);
@@ -148,9 +155,11 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
 #pragma unroll
                     for (int t = 0; t < 16; ++t) {
                         const float s = T::to_f32(sv[t]);
+                        const float sb = -T::kBias * s;  // exact: a power of two plus a small multiple times a 16-bit float
 #pragma unroll
                         for (int v = 0; v < 4; ++v) {
-                            total[t][v] += (acc[t][v] - T::kBias * xsum[v]) * s;
+                            total[t][v] = fmaf(acc[t][v], s, total[t][v]);
+                            total[t][v] = fmaf(xsum[v], sb, total[t][v]);
                             acc[t][v] = 0.f;
                         }
                     }
@@ -229,7 +238,11 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
             launch(kern, dim3(grid), dim3(256), shmem, stream, ap0 + m0 * lda, lda, wp, sp, cp0 + m0 * n, mt, int(k), int(n),
                    group, rpb, splits, tiles, partials, counters);
         };
-        if (dtype == HIDET_QMM_F16) {
+        const bool full = aligned_a && n % kSkinnyTileN == 0 && k % rpb == 0 && rpb % (kSkinnyWaves * 64) == 0;
+        if (full) {
+            if (dtype == HIDET_QMM_F16) go(skinny_w4a16_kernel<HIDET_QMM_F16, 2, true, true>);
+            else go(skinny_w4a16_kernel<HIDET_QMM_BF16, 2, true, true>);
+        } else if (dtype == HIDET_QMM_F16) {
             if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, 2, true>);
             else go(skinny_w4a16_kernel<HIDET_QMM_F16, 2, false>);
         } else {
