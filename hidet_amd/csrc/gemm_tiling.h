@@ -251,6 +251,35 @@ inline GemmTail make_gemm_tail(const GemmTiling &t, int concurrent, int fill, in
     return tail;
 }
 
+// The same decision by counting rounds: with `concurrent` workgroup slots per XCD, the busiest XCD needs
+// floor(n / concurrent) whole rounds plus ceil(rest * parts / concurrent) / parts of a round for its `rest` tail tiles
+// cut into `parts` K ranges; the exchange of the partial tiles moves 8 * rest * parts tiles' worth of accumulators
+// through memory, `exchange_cost` of a tile's compute time each (all workgroups share the memory system, so this adds
+// up chip-wide). Takes the part count that minimises the sum if it saves at least a tenth of a round. Unlike
+// make_gemm_tail this also splits a short tail behind whole rounds (33 tiles on 32 slots: 2 rounds -> 1.3), and does
+// not split when that only trades one long round for several short ones of the same total (22 tiles on 32 slots: 2 or
+// 3 parts change nothing, 4 parts save a quarter round but their exchange costs more than that).
+inline GemmTail make_gemm_tail_by_rounds(const GemmTiling &t, int concurrent, int max_parts, double exchange_cost) {
+    GemmTail tail{1, 0, t.grid()};
+    int busiest = 0;
+    for (int x = 0; x < 8; ++x) {
+        const int n = gemm_region_tiles(t, x);
+        if (n > busiest) busiest = n;
+        if (n % concurrent > tail.max_tiles) tail.max_tiles = n % concurrent;
+    }
+    const int rest = busiest % concurrent;
+    if (rest == 0) return tail;
+    double best = 1.0;
+    for (int p = 2; p <= max_parts; ++p) {
+        const double rounds = double((rest * p + concurrent - 1) / concurrent) / p + 8.0 * rest * p * exchange_cost;
+        if (rounds < best - 0.1) {
+            best = rounds;
+            tail.parts = p;
+        }
+    }
+    return tail;
+}
+
 // Workgroups per XCD x 8 once the tails are cut into tail.parts ranges.
 inline int64_t gemm_grid_with_tail(const GemmTiling &t, int concurrent, const GemmTail &tail) {
     if (tail.parts <= 1) return t.grid();
