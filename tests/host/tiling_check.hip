@@ -9,11 +9,17 @@
 
 using namespace qmm;
 
-static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_parts, bool tile_only) {
+// mode 0: the planner by fill; 1: no K ranges; 2: the planner by rounds (fill = the exchange cost in 1e-4 of a tile's time)
+static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_parts, int mode) {
     const GemmTiling t = make_gemm_tiling(tiles_m, tiles_n, concurrent);
     if (t.xm * t.xn != 8) return std::printf("tiling %dx%d: %d x %d regions\n", tiles_m, tiles_n, t.xm, t.xn), 1;
     GemmTail tail = make_gemm_tail(t, concurrent, fill, max_parts);
-    if (tile_only) tail = GemmTail{1, 0, t.grid()};
+    if (mode == 1) tail = GemmTail{1, 0, t.grid()};
+    if (mode == 2) {
+        tail = make_gemm_tail_by_rounds(t, concurrent, max_parts, fill * 1e-4);
+        if (tail.parts < 1 || tail.parts > max_parts || tail.max_tiles >= concurrent)
+            return std::printf("%dx%d c%d: plan by rounds gives %d parts, %d tail tiles\n", tiles_m, tiles_n, concurrent, tail.parts, tail.max_tiles), 1;
+    }
     const long long grid = gemm_grid_with_tail(t, concurrent, tail);
     std::vector<int> seen(size_t(tiles_m) * tiles_n * max_parts, 0), parts_of(size_t(tiles_m) * tiles_n, 0);
     std::vector<int> slot_owner(size_t(8) * (tail.max_tiles > 0 ? tail.max_tiles : 1), -1);
@@ -81,9 +87,11 @@ int main() {
     for (const auto &c : cfgs)
         for (int tm = 1; tm <= 70; tm += (tm < 20 ? 1 : 7))
             for (int tn = 1; tn <= 130; tn += (tn < 50 ? 1 : 9)) {
-                if (check(tm, tn, c[0], c[1], c[2], false)) return 1;
-                if (check(tm, tn, c[0], c[1], c[2], true)) return 1;
-                n += 2;
+                if (check(tm, tn, c[0], c[1], c[2], 0)) return 1;
+                if (check(tm, tn, c[0], c[1], c[2], 1)) return 1;
+                if (check(tm, tn, c[0], 7, c[2], 2)) return 1;
+                if (check(tm, tn, c[0], 0, c[2], 2)) return 1;  // free exchange: splits wherever a round is partly filled
+                n += 4;
             }
     std::printf("ok %lld launches\n", n);
     return 0;
