@@ -267,17 +267,26 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     // (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
     // (light workgroups - at most 4 active row blocks - are worth up to 8 ranges: measured)
     GemmTail tail = make_gemm_tail(tiling, kConcurrent, 32, RBA <= 4 ? 8 : 4);
+    // Full tiles: count rounds of one workgroup per CU. The tiles past a whole number of such rounds share their CUs
+    // with another workgroup or run in a round of their own; cut into K ranges they finish sooner when they are few
+    // (K = 4096, N = 11008: M = 768 / 896 / 1024: 96 / 94.5 / 96 -> 88 / 84 / 91.5 us, M = 1536 / 1792: 149.5 / 153 -> 133 /
+    // 140 us; up to 8 ranges instead of 4: no further gain).
+    int split_unit = kConcurrent;
+    if (RBA == 8 && tail.parts == 1) {
+        tail = make_gemm_tail_by_rounds(tiling, 32, 4, 0.00085 * 4096.0 / double(k));
+        split_unit = 32;
+    }
     while (tail.parts > 1 &&
            (k / kBK < 8 * tail.parts ||
             workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
         --tail.parts;
     static_assert(8 * kConcurrent * 4 <= kCounterBytes, "one counter per tail tile");
-    const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
+    const int64_t grid = gemm_grid_with_tail(tiling, split_unit, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
     allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>), Cfg::kLdsBytes);
     launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale),
-           static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent, tail.parts, tail.max_tiles,
+           static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, split_unit, tail.parts, tail.max_tiles,
            reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
 }
 
