@@ -9,13 +9,14 @@
 
 using namespace qmm;
 
-// mode 0: the planner by fill; 1: no K ranges; 2: the planner by rounds (fill = the exchange cost in 1e-4 of a tile's time)
+// mode 0: the planner by fill; 1: no K ranges; 2: the planner by rounds (fill = the exchange cost in 1e-4 of a tile's time);
+// 3: as 2 with the regions laid out for twice as many workgroups at a time as the rounds are counted in (two per CU)
 static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_parts, int mode) {
-    const GemmTiling t = make_gemm_tiling(tiles_m, tiles_n, concurrent);
+    const GemmTiling t = make_gemm_tiling(tiles_m, tiles_n, mode == 3 ? 2 * concurrent : concurrent);
     if (t.xm * t.xn != 8) return std::printf("tiling %dx%d: %d x %d regions\n", tiles_m, tiles_n, t.xm, t.xn), 1;
     GemmTail tail = make_gemm_tail(t, concurrent, fill, max_parts);
     if (mode == 1) tail = GemmTail{1, 0, t.grid()};
-    if (mode == 2) {
+    if (mode >= 2) {
         tail = make_gemm_tail_by_rounds(t, concurrent, max_parts, fill * 1e-4);
         if (tail.parts < 1 || tail.parts > max_parts || tail.max_tiles >= concurrent)
             return std::printf("%dx%d c%d: plan by rounds gives %d parts, %d tail tiles\n", tiles_m, tiles_n, concurrent, tail.parts, tail.max_tiles), 1;
@@ -91,7 +92,8 @@ int main() {
                 if (check(tm, tn, c[0], c[1], c[2], 1)) return 1;
                 if (check(tm, tn, c[0], 7, c[2], 2)) return 1;
                 if (check(tm, tn, c[0], 0, c[2], 2)) return 1;  // free exchange: splits wherever a round is partly filled
-                n += 4;
+                if (check(tm, tn, c[0], 2, c[2], 3)) return 1;
+                n += 5;
             }
     std::printf("ok %lld launches\n", n);
     return 0;
