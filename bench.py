@@ -327,6 +327,10 @@ def main():
         nbytes = K * N // 2 + 2 * (K // 128) * N + 2 * m4 * K + 2 * m4 * N
         others['w4a16_m{}_k4096_n11008'.format(m4)] = (hbm_entry(us, nbytes) if m4 <= 16 else
                                                       mfma_entry(us, 2.0 * m4 * K * N, MFMA_F16_PEAK_TFLOPS))
+        if m4 <= 16:  # the same bytes read as the [N, K/2] decode layout (another data layout: never the headline)
+            us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16_nk', a4, w4[r % 16].view(N, K // 2), s4, c4, m4, K, N,
+                                              K, K // 2, 128, 2, sptr), 40, 16)
+            others['w4a16_m{}_k4096_n11008_decode_layout'.format(m4)] = hbm_entry(us, nbytes)
     del w4
     # FP8 decode variant: M = 1 against the same b
     a1 = a8[:1].contiguous()

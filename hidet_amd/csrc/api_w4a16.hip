@@ -9,6 +9,9 @@ bool gemm_w4a16_supported(const void *a, const void *w, const void *scales, cons
                           int64_t lda, int group);
 void gemm_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, int group, int dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+bool skinny_w4a16_nk_supported(const void *a, const void *w, int64_t k, int64_t lda, int64_t ldw, int group);
+void skinny_w4a16_nk_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
+                            int64_t lda, int64_t ldw, int group, int dtype, hipStream_t stream);
 }  // namespace qmm
 
 using namespace qmm;
@@ -37,5 +40,26 @@ HIDET_API void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, 
     else
         skinny_w4a16_launch(a, w, scales, c, m, k, n, lda, group_size, dtype, parallel_k_parts, workspace, workspace_bytes,
                             stream);
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_symmetric_quant_matmul_w4a16_nk(const void *a, const void *w_nk, const void *scales, void *c, int64_t m,
+                                                     int64_t k, int64_t n, int64_t lda, int64_t ldw, int group_size, int dtype,
+                                                     void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(dtype == HIDET_QMM_BF16 || dtype == HIDET_QMM_F16,
+              "activations and scales must be bfloat16 or float16, got dtype code " << dtype);
+    QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
+    QMM_CHECK(group_size > 0 && k % group_size == 0,
+              "K (" << k << ") must be a multiple of the group size (" << group_size << ")");
+    QMM_CHECK(lda >= k, "row stride of a (" << lda << ") is smaller than K (" << k << ")");
+    QMM_CHECK(2 * ldw >= k, "row stride of w_nk (" << ldw << " bytes) is smaller than K / 2 (" << k / 2 << ")");
+    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    if (m == 0 || n == 0) return;
+    QMM_CHECK(a && c && w_nk && scales, "null tensor pointer");
+    QMM_CHECK(skinny_w4a16_nk_supported(a, w_nk, k, lda, ldw, group_size),
+              "the K-contiguous int4 kernel needs K a multiple of 128, a group size of 128 times a power of two, 16-byte "
+              "aligned rows of w_nk and of a: k=" << k << " group=" << group_size << " lda=" << lda << " ldw=" << ldw);
+    skinny_w4a16_nk_launch(a, w_nk, scales, c, m, k, n, lda, ldw, group_size, dtype, static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

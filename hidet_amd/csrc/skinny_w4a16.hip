@@ -11,32 +11,10 @@
 // of a 16x16x32 MFMA.  The constant is removed per group with one extra MFMA against ones; at every group
 // boundary the fp32 accumulators are scaled into the running totals.
 #include "skinny_common.h"
+#include "w4_traits.h"
 
 namespace qmm {
 namespace {
-
-template <int DT>
-struct W4Traits;
-template <>
-struct W4Traits<HIDET_QMM_BF16> {
-    static constexpr uint32_t kMagic = 0x43084308u;
-    static constexpr float kBias = 136.0f;
-    static constexpr uint16_t kOne = 0x3F80;
-    static __device__ __forceinline__ float4_t mfma(const uint4 &a, const uint4 &b, float4_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ float to_f32(uint16_t b) { return bf16_bits_to_f32(b); }
-};
-template <>
-struct W4Traits<HIDET_QMM_F16> {
-    static constexpr uint32_t kMagic = 0x64086408u;
-    static constexpr float kBias = 1032.0f;
-    static constexpr uint16_t kOne = 0x3C00;
-    static __device__ __forceinline__ float4_t mfma(const uint4 &a, const uint4 &b, float4_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ float to_f32(uint16_t b) { return f16_bits_to_f32(b); }
-};
 
 template <int DT, int DEPTH, bool ALIGNED_A, bool FULL = false>
 __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,

@@ -95,3 +95,52 @@ def symmetric_quant_matmul_w4a16(a: torch.Tensor, packed: torch.Tensor, scales: 
     if len(a.shape) < 2 or len(packed.shape) < 2:
         raise ValueError('a and b must have at least 2 dimensions, got shape {} and {}'.format(list(a.shape), list(packed.shape)))
     return SymmetricQuantizedMatmulW4A16Op(a, packed, scales, group_size).outputs[0]
+
+
+def to_decode_layout_int4(packed: torch.Tensor) -> torch.Tensor:
+    """Repack `packed` uint8 [K, N/2] (two codes per byte along N, low nibble first) as uint8 [N, K/2] for the decode kernel.
+
+    Row n of the result holds the K codes of output column n; inside every 4 bytes (8 consecutive k) nibble i is code
+    k = 2i for i < 4 and code k = 2(i - 4) + 1 for i >= 4, so that a shift and a mask give the kernel a (k, k + 1) pair
+    ready for the matrix instruction. K must be a multiple of 8 (the kernel itself wants 128).
+    """
+    if packed.dim() != 2 or packed.dtype != torch.uint8:
+        raise ValueError('expected a packed uint8 weight [K, N/2], got {} {}'.format(packed.dtype, list(packed.shape)))
+    k, n = packed.shape[0], packed.shape[1] * 2
+    if k % 8 != 0:
+        raise ValueError('K ({}) must be a multiple of 8'.format(k))
+    codes = torch.stack((packed & 0xF, packed >> 4), dim=-1).reshape(k, n)   # nibble of q[k, n]
+    pairs = codes.t().reshape(n, k // 8, 4, 2)                                # [n, word, i, parity]: code k = 2i + parity
+    even, odd = pairs[..., 0], pairs[..., 1]
+    out = torch.stack((even[..., 0] | (even[..., 1] << 4), even[..., 2] | (even[..., 3] << 4),
+                       odd[..., 0] | (odd[..., 1] << 4), odd[..., 2] | (odd[..., 3] << 4)), dim=-1)
+    return out.reshape(n, k // 2).contiguous()
+
+
+def symmetric_quant_matmul_w4a16_decode(a: torch.Tensor, packed_nk: torch.Tensor, scales: torch.Tensor,
+                                        group_size: int = 128) -> torch.Tensor:
+    """`symmetric_quant_matmul_w4a16` on a weight repacked with `to_decode_layout_int4` ([N, K/2]); `scales` stay
+    [K/group, N]. For decode: up to 16 rows of `a` per pass over the weights. K a multiple of 128, group size 128 times
+    a power of two."""
+    if len(a.shape) < 2 or len(packed_nk.shape) != 2 or len(scales.shape) != 2:
+        raise ValueError('expect a[..., M, K], packed_nk[N, K/2], scales[K/g, N], got {}, {} and {}'.format(
+            list(a.shape), list(packed_nk.shape), list(scales.shape)))
+    if a.dtype not in (torch.bfloat16, torch.float16) or scales.dtype != a.dtype or packed_nk.dtype != torch.uint8:
+        raise ValueError('Expect a and scales to be bfloat16 or float16 (same type) and the packed weight to be uint8')
+    n, k = packed_nk.shape[0], packed_nk.shape[1] * 2
+    if a.shape[-1] != k:
+        raise ValueError('Matrix multiplication expect tensor A and B with shape [..., M, K] and [..., K, N]'
+                         ', got {} and {}'.format(list(a.shape), [k, n]))
+    if group_size <= 0 or k % group_size != 0 or tuple(scales.shape) != (k // group_size, n):
+        raise ValueError('scales must be [K / group, N] = {}, got {}'.format([k // max(group_size, 1), n], list(scales.shape)))
+    ffi.require_gpu(a, packed_nk, scales)
+    a2 = a.reshape(-1, k)
+    if a2.stride(-1) != 1 or (a2.shape[0] > 1 and (a2.stride(0) < k or a2.stride(0) % 8 != 0)) or a2.data_ptr() % 16 != 0:
+        a2 = a2.contiguous()
+    m = a2.shape[0]
+    lda = a2.stride(0) if m > 1 else k
+    c = torch.empty((m, n), dtype=a.dtype, device=a.device)
+    packed_nk = packed_nk.contiguous()
+    ffi.call('hidet_symmetric_quant_matmul_w4a16_nk', a2, packed_nk, scales.contiguous(), c, m, k, n, lda, k // 2, group_size,
+             ffi.DTYPE_CODE[a.dtype], ffi.current_stream(a.device))
+    return c.reshape(tuple(a.shape[:-1]) + (n,))

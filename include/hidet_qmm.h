@@ -112,6 +112,16 @@ void hidet_group_quantize_int4(const void *w, void *packed, void *scales, int64_
 void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k,
                                         int64_t n, int64_t lda, int group_size, int dtype, int parallel_k_parts,
                                         void *workspace, int64_t workspace_bytes, void *stream);
+/* The same operator on weights repacked for decode: w_nk is uint8 [n, k/2] with row stride ldw bytes, row n holding
+ * the k codes of output column n; inside every 32-bit word (8 consecutive k) nibble i is code 2i for i < 4 and code
+ * 2(i-4)+1 for i >= 4 (hidet_amd.graph.ops.quant.to_decode_layout_int4 repacks). scales stay [k/group, n]. No
+ * counterpart in the reference, like the operator itself; the layout is the int4 analogue of the transpose_b=True
+ * weight of python/hidet/graph/ops/matmul/matmul.py:37-38. Needs k a multiple of 128, a group size of 128 times a
+ * power of two and 16-byte aligned rows; meant for decode: every 16 rows of a are one more pass over the weights.
+ * No workspace. */
+void hidet_symmetric_quant_matmul_w4a16_nk(const void *a, const void *w_nk, const void *scales, void *c, int64_t m,
+                                           int64_t k, int64_t n, int64_t lda, int64_t ldw, int group_size, int dtype,
+                                           void *stream);
 
 /* ---- per-tensor float8 e4m3 quantization (benchmark configuration) --------------------------------
  * scale[0] = max|x| / 448 (float32, written to device memory), codes = e4m3(x / scale), round to nearest

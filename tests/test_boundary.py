@@ -159,3 +159,22 @@ def test_header_is_plain_c():
     r = subprocess.run([gcc, '-std=c99', '-Wall', '-Werror', '-fsyntax-only', '-x', 'c', os.path.join(ROOT, 'include', 'hidet_qmm.h')],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout
+
+
+def test_int4_decode_layout_repacking():
+    # to_decode_layout_int4 is host logic (torch ops only): nibble i of every 32-bit word of row n is code k = 2i for
+    # i < 4 and k = 2(i - 4) + 1 for i >= 4 of column n
+    import numpy as np
+    import torch
+    from hidet_amd.graph.ops.quant import to_decode_layout_int4
+    rng = np.random.default_rng(0)
+    k, n = 64, 10
+    u = (rng.integers(-8, 8, (k, n)) & 0xF).astype(np.uint8)
+    packed = (u[:, 0::2] | (u[:, 1::2] << 4)).astype(np.uint8)
+    words = to_decode_layout_int4(torch.from_numpy(packed)).numpy().view('<u4')
+    assert words.shape == (n, k // 8)
+    for i in range(8):
+        kk = np.arange(k // 8) * 8 + (2 * i if i < 4 else 2 * (i - 4) + 1)
+        assert np.array_equal((words >> np.uint32(4 * i)) & 0xF, u[kk].T)
+    with pytest.raises(ValueError):
+        to_decode_layout_int4(torch.zeros(12, 4, dtype=torch.uint8))

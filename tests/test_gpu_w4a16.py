@@ -89,6 +89,50 @@ def test_exact_on_small_integers():
         assert np.array_equal(got, O.to_bf16(want.astype(np.float32))), (m, k, n)
 
 
+@pytest.mark.parametrize('m,k,n,g', [(1, 4096, 11008, 128), (16, 4096, 11008, 128), (2, 1024, 4096, 256), (5, 384, 40, 128),
+                                     (9, 1152, 72, 128), (3, 128, 16, 128), (21, 2048, 528, 1024), (1, 11008 - 11008 % 128, 4096, 128)])
+@pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
+def test_decode_layout_parity_and_same_result_as_row_major(m, k, n, g, dtype):
+    # the weight repacked K-contiguous for decode: same operator, compared with the oracle and with the row-major kernels
+    # (4 and 8 waves, direct and LDS-staged activations, waves with an empty K range, a second 16-row pass, groups of
+    # several steps)
+    announce('w4a16 decode layout', m, k, n, g, dtype)
+    a, packed, scales, ta, tp, ts = _case(m * 13 + n, m, k, n, g, dtype)
+    tp_nk = quant.to_decode_layout_int4(tp)
+    assert tuple(tp_nk.shape) == (n, k // 2) and tp_nk.is_contiguous()
+    got = host(quant.symmetric_quant_matmul_w4a16_decode(ta, tp_nk, ts, g))
+    ref = O.w4a16_matmul(a, packed, scales, g, dtype)
+    err = O.max_rel_err(got, ref)
+    assert err <= TOL, err
+    other = host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g))
+    assert O.max_rel_err(got, other) <= 1e-2
+
+
+def test_decode_layout_exact_and_errors():
+    announce('w4a16 decode layout exact')
+    rng = np.random.default_rng(11)
+    for m, k, n, g in ((1, 256, 32, 128), (4, 1280, 8200, 256), (16, 4096, 64, 128)):
+        a = rng.integers(-4, 5, (m, k)).astype(np.float32)
+        q = rng.integers(-7, 8, (k, n)).astype(np.int8)
+        s = np.exp2(rng.integers(-3, 2, (k // g, n))).astype(np.float32)
+        packed = O.pack_int4(q)
+        want = np.zeros((m, n), np.float64)
+        for gi in range(k // g):
+            want += (a[:, gi * g:(gi + 1) * g].astype(np.float64) @ q[gi * g:(gi + 1) * g].astype(np.float64)) * s[gi][None, :]
+        tp_nk = quant.to_decode_layout_int4(dev(packed))
+        got = quant.symmetric_quant_matmul_w4a16_decode(dev(a, torch.bfloat16), tp_nk, dev(s, torch.bfloat16), g)
+        assert np.array_equal(host(got), O.to_bf16(want.astype(np.float32))), (m, k, n)
+    import hidet_amd
+    with pytest.raises(hidet_amd.BackendException, match='multiple of 128'):
+        quant.symmetric_quant_matmul_w4a16_decode(torch.zeros(1, 64, device='cuda', dtype=torch.bfloat16),
+                                                  torch.zeros(16, 32, device='cuda', dtype=torch.uint8),
+                                                  torch.zeros(1, 16, device='cuda', dtype=torch.bfloat16), 64)
+    with pytest.raises(ValueError, match='scales must be'):
+        quant.symmetric_quant_matmul_w4a16_decode(torch.zeros(1, 128, device='cuda', dtype=torch.bfloat16),
+                                                  torch.zeros(16, 64, device='cuda', dtype=torch.uint8),
+                                                  torch.zeros(2, 16, device='cuda', dtype=torch.bfloat16), 128)
+
+
 def test_k_split_is_deterministic():
     m, k, n, g = 129, 4096, 512, 128
     announce('w4a16 k split twice', m, k, n)
