@@ -32,6 +32,9 @@ def test_w8a16_random_shapes_exact(seed):
         want = (a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :]
         got = host(quant.symmetric_quant_matmul(dev(a), dev(q), dev(s)))
         assert np.array_equal(got, want.astype(np.float32).astype(np.float16)), (m, k, n)
+        # the same weight stored K-contiguous: up to 16 rows run the kernels for that layout, more rows a row-major copy
+        got = host(quant.symmetric_quant_matmul(dev(a), quant.to_decode_layout(dev(q)), dev(s)))
+        assert np.array_equal(got, want.astype(np.float32).astype(np.float16)), ('k-contiguous', m, k, n)
 
 
 @pytest.mark.parametrize('seed', range(4))
@@ -54,6 +57,10 @@ def test_w4a16_random_shapes_exact(seed, dtype):
         got = host(quant.symmetric_quant_matmul_w4a16(dev(a, tdt), dev(O.pack_int4(q)), dev(scales, tdt), g))
         exp = O.to_bf16(want.astype(np.float32)) if dtype == 'bfloat16' else want.astype(np.float32).astype(np.float16)
         assert np.array_equal(got, exp), (m, k, n, g)
+        if k % 128 == 0 and g == 128 and m <= 40:  # the decode layout of the same codes
+            nk = quant.to_decode_layout_int4(dev(O.pack_int4(q)))
+            got = host(quant.symmetric_quant_matmul_w4a16_decode(dev(a, tdt), nk, dev(scales, tdt), g))
+            assert np.array_equal(got, exp), ('decode layout', m, k, n, g)
 
 
 @pytest.mark.parametrize('seed', range(5))
