@@ -29,6 +29,22 @@ def _w4(m, k, n):
     return a, (lambda x: quant.symmetric_quant_matmul_w4a16(x, w, s, 128))
 
 
+def _w8_nk(m, k, n):
+    g = torch.Generator(device='cuda').manual_seed(m * 17 + n)
+    a = torch.randn(m, k, device='cuda', generator=g).half()
+    w = quant.to_decode_layout(torch.randint(-127, 128, (k, n), device='cuda', dtype=torch.int8, generator=g))
+    s = (torch.rand(n, device='cuda', generator=g) * 0.01).half()
+    return a, (lambda x: quant.symmetric_quant_matmul(x, w, s))
+
+
+def _w4_nk(m, k, n):
+    g = torch.Generator(device='cuda').manual_seed(m * 19 + n)
+    a = torch.randn(m, k, device='cuda', generator=g).bfloat16()
+    w = quant.to_decode_layout_int4(torch.randint(0, 256, (k, n // 2), device='cuda', dtype=torch.uint8, generator=g))
+    s = (torch.rand(k // 128, n, device='cuda', generator=g) * 0.01).bfloat16()
+    return a, (lambda x: quant.symmetric_quant_matmul_w4a16_decode(x, w, s, 128))
+
+
 def _f8(m, k, n):
     g = torch.Generator(device='cuda').manual_seed(m * 13 + n)
     a = torch.randint(0, 0x7F, (m, k), device='cuda', dtype=torch.uint8, generator=g).view(torch.float8_e4m3fn)
@@ -38,7 +54,8 @@ def _f8(m, k, n):
 
 CASES = [('w8a16 gemv, K slices', _w8, 1, 4096, 1024), ('w8a16 gemm, K ranges of short tiles', _w8, 48, 4096, 1024),
          ('w8a16 16 rows', _w8, 16, 4096, 512), ('w4a16 gemv', _w4, 1, 4096, 1024), ('w4a16 gemm, K ranges', _w4, 129, 4096, 512),
-         ('fp8 gemm, K ranges', _f8, 100, 8192, 1024)]
+         ('fp8 gemm, K ranges', _f8, 100, 8192, 1024), ('fp8 16 rows', _f8, 16, 4096, 1024),
+         ('w8a16 decode layout', _w8_nk, 8, 4096, 1024), ('w4a16 decode layout', _w4_nk, 8, 4096, 1024)]
 
 
 @pytest.mark.parametrize('name,make,m,k,n', CASES, ids=[c[0] for c in CASES])
