@@ -118,9 +118,14 @@ def main():
             for rep in range(2):
                 for i in range(RING):
                     launch(i, sptr)
+            # the same ring read as K-contiguous [N, K] weights by the kernel for that layout (other_configs)
+            c_nk = torch.empty((1, N), dtype=torch.float16, device=device)
+            for rep in range(2):
+                for i in range(RING):
+                    ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a, ws[i].view(N, K), ss[0], c_nk, 1, K, N, K, K, sptr)
         stream.synchronize()
         print(json.dumps({'pmc_calibration': {'copy_bytes': 64 << 20, 'copies': 4, 'gemv_launches': 2 * RING,
-                                              'gemv_algorithmic_bytes': GEMV_BYTES}}))
+                                              'gemv_k_contiguous_launches': 2 * RING, 'gemv_algorithmic_bytes': GEMV_BYTES}}))
         return
 
     # ---- parity of one ring entry against the oracle, before anything is timed --------------------------
