@@ -10,6 +10,8 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
                      hipStream_t stream);
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
                             int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+void skinny_fp8_block_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
+                                    int64_t n, int64_t k, int out_dtype, hipStream_t stream);
 }  // namespace qmm
 
 using namespace qmm;
@@ -59,6 +61,9 @@ HIDET_API void hidet_matmul_f8_scaled(const void *a, const void *b, const void *
     QMM_CHECK(k > 0, "K must be positive");
     QMM_CHECK(aligned(a, 16) && aligned(b, 16) && aligned(c, 16), "tensors must be 16-byte aligned");
     check_workspace(workspace, workspace_bytes);
-    gemm_fp8_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
+    if (m <= 16)  // decode: the bandwidth-bound kernel, one pass over b
+        skinny_fp8_block_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, static_cast<hipStream_t>(stream_));
+    else
+        gemm_fp8_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

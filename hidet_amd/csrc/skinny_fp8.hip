@@ -105,7 +105,11 @@ __global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restri
 // with two fully coalesced loads (8 rows x 128 bytes each) and reads its operand back from a private LDS tile of
 // 16 rows x (128 + 16) bytes, two slots; no barrier, one wave's LDS operations execute in order.  The loop has no
 // conditions: lanes of rows >= M and columns >= N read a clamped row and their results are dropped.
-template <int OUT, int WAVES>
+// BLOCK_SCALED: scale_a is [K / 128, M] and scale_b [N / 128, K / 128] (one factor per 128-deep step and row, and per step
+// and 128 output columns): every step's products are accumulated from zero and added to the total times both factors.
+// The 16 row factors of a step are fetched by the 16 lanes of a group like one more operand and turned into the four
+// each lane needs (rows 4 kg .. 4 kg + 3) through LDS, per step, as the activations are.
+template <int OUT, int WAVES, bool BLOCK_SCALED = false>
 __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uint8_t *__restrict__ a, int64_t lda,
                                                                 const uint8_t *__restrict__ b, int64_t ldb,
                                                                 void *__restrict__ c, int m, int n, int k,
@@ -113,6 +117,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
                                                                 const float *__restrict__ scale_b) {
     __shared__ float red[WAVES][16][17];
     __shared__ uint4 stage[WAVES][2][16 * 9];
+    __shared__ float4_t factor_stage[BLOCK_SCALED ? WAVES : 1][2][4];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 4, ls = lane & 15;
@@ -123,17 +128,22 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
     const int s_begin = wave * steps_per_wave, s_end = min(steps, s_begin + steps_per_wave);
 
     float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    const float *sa_col = BLOCK_SCALED ? scale_a + min(ls, m - 1) : nullptr;
+    const float *sb_row = BLOCK_SCALED ? scale_b + int64_t(n0 >> 7) * steps : nullptr;  // 16 columns lie in one 128-column block
     const uint8_t *bp = b + int64_t(min(n0 + ls, n - 1)) * ldb + 32 * kg;
     const uint8_t *ap0 = a + int64_t(min(lane >> 3, m - 1)) * lda + 16 * (lane & 7);
     const uint8_t *ap1 = a + int64_t(min(8 + (lane >> 3), m - 1)) * lda + 16 * (lane & 7);
 
     for (int s0 = s_begin; s0 < s_end; s0 += kDepth) {
         uint4 wv[kDepth][2], ax[kDepth][2];
+        float fr[BLOCK_SCALED ? kDepth : 1];
 #pragma unroll
         for (int d = 0; d < kDepth; ++d) {
             const int st = min(s0 + d, s_end - 1);  // a step past the wave's range re-reads its last one; not used
             wv[d][0] = *reinterpret_cast<const uint4 *>(bp + int64_t(st) * 128);
             wv[d][1] = *reinterpret_cast<const uint4 *>(bp + int64_t(st) * 128 + 16);
+            if (BLOCK_SCALED) fr[d] = sa_col[int64_t(st) * m] * sb_row[st];
         }
 #pragma unroll
         for (int d = 0; d < kDepth; ++d) {
@@ -143,7 +153,11 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
         }
 #pragma unroll
         for (int d = 0; d < kDepth; ++d) {
-            if (s0 + d >= s_end) break;  // wave-uniform
+            // One block per step (wave-uniform branch): the compiler moves each step's loads down into its block, so a
+            // wave has one step in flight at a time and the many waves per CU hide the latency.  Measured against the
+            // same loop without the branch, where all eight steps' loads really are issued up front: 8192 x 8192, one
+            // row: 12 us against 18 us.
+            if (s0 + d >= s_end) break;
             uint4 *tile = stage[wave][d & 1];
             tile[(lane >> 3) * 9 + (lane & 7)] = ax[d][0];
             tile[(8 + (lane >> 3)) * 9 + (lane & 7)] = ax[d][1];
@@ -153,7 +167,16 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
             rv[4] = int(x1.x); rv[5] = int(x1.y); rv[6] = int(x1.z); rv[7] = int(x1.w);
             cv[0] = int(wv[d][0].x); cv[1] = int(wv[d][0].y); cv[2] = int(wv[d][0].z); cv[3] = int(wv[d][0].w);
             cv[4] = int(wv[d][1].x); cv[5] = int(wv[d][1].y); cv[6] = int(wv[d][1].z); cv[7] = int(wv[d][1].w);
-            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+            if (BLOCK_SCALED) {
+                float *ft = reinterpret_cast<float *>(factor_stage[wave][d & 1]);
+                ft[ls] = fr[d];  // the four lane groups store the same 16 values
+                const float4_t f = factor_stage[wave][d & 1][kg];
+                const float4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, zero, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = fmaf(part[v], f[v], acc[v]);
+            } else {
+                acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+            }
         }
     }
 #pragma unroll
@@ -164,8 +187,8 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
         float v = 0.f;
 #pragma unroll
         for (int p = 0; p < WAVES; ++p) v += red[p][row][cn];
-        if (scale_a != nullptr) v *= *scale_a;
-        if (scale_b != nullptr) v *= *scale_b;
+        if (!BLOCK_SCALED && scale_a != nullptr) v *= *scale_a;
+        if (!BLOCK_SCALED && scale_b != nullptr) v *= *scale_b;
         const int64_t o = int64_t(row) * n + n0 + cn;
         if (OUT == HIDET_QMM_F32) static_cast<float *>(c)[o] = v;
         else if (OUT == HIDET_QMM_BF16) static_cast<uint16_t *>(c)[o] = f32_to_bf16_bits(v);
@@ -203,6 +226,30 @@ void skinny_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t
         default: QMM_FAIL("unsupported output dtype code " << out_dtype);
     }
 #undef QMM_FP8_SKINNY
+}
+
+// Block-scaled operands (scale_a f32 [K/128, M], scale_b f32 [N/128, K/128]), up to 16 rows, contiguous a [M, K] and b [N, K],
+// K and N multiples of 128, everything 16-byte aligned (the entry point checks that).
+void skinny_fp8_block_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
+                                    int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+    const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
+    const float *sa = static_cast<const float *>(scale_a), *sb = static_cast<const float *>(scale_b);
+    const dim3 grid(uint32_t(cdiv(n, 16)));
+    const bool eight = cdiv(n, 16) < kEightWaveTiles && k >= 8 * 128;
+    auto go = [&](auto kern, int waves) {
+        launch(kern, grid, dim3(64 * waves), 0, stream, ap, k, bp, k, c, int(m), int(n), int(k), sa, sb);
+    };
+#define QMM_FP8_SKINNY_SCALED(OUT)                                          \
+    if (eight) go(skinny_fp8_staged_kernel<OUT, 8, true>, 8);               \
+    else go(skinny_fp8_staged_kernel<OUT, 4, true>, 4);
+    switch (out_dtype) {
+        case HIDET_QMM_F32: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F32) break;
+        case HIDET_QMM_F16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F16) break;
+        case HIDET_QMM_BF16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_BF16) break;
+        case HIDET_QMM_E4M3: QMM_FP8_SKINNY_SCALED(HIDET_QMM_E4M3) break;
+        default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+    }
+#undef QMM_FP8_SKINNY_SCALED
 }
 
 }  // namespace qmm

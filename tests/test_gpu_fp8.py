@@ -102,7 +102,10 @@ def test_matmul_f8_reference_recipe(a_shape, b_shape):
 
 @pytest.mark.parametrize('a_shape, b_shape', [[[4096, 4096], [4096, 4096]], [[2048, 256], [4096, 256]], [[100, 384], [256, 384]],
                                               [[16384, 7168], [1536, 7168]],
-                                              [[40, 4096], [1024, 4096]], [[130, 2048], [512, 2048]], [[500, 7168], [1536, 7168]]])  # K ranges
+                                              [[40, 4096], [1024, 4096]], [[130, 2048], [512, 2048]], [[500, 7168], [1536, 7168]],  # K ranges
+                                              # up to 16 rows: the bandwidth-bound kernel, 8 and 4 waves per workgroup
+                                              [[1, 7168], [1536, 7168]], [[16, 4096], [4096, 4096]], [[5, 384], [256, 384]],
+                                              [[9, 2048], [8192, 2048]], [[3, 128], [128, 128]]])
 def test_matmul_f8_scaled_reference_recipe(a_shape, b_shape):
     # tests/operators_core/test_matmul.py:291-373: integers in [-5, 4], integer scales 1..4, bf16 output; the
     # expected value is built by pre-multiplying the scales into the operands (exact in int64)
@@ -125,6 +128,22 @@ def test_matmul_f8_scaled_reference_recipe(a_shape, b_shape):
     if m <= 128:
         ref = O.matmul_f8_scaled(O.e4m3_encode(ai.astype(np.float32)), O.e4m3_encode(bi.astype(np.float32)), sa, sb, 'float32')
         assert np.array_equal(host(got), ref)
+
+
+@pytest.mark.parametrize('m,k,n', [(1, 4096, 4096), (7, 7168, 1536), (16, 2048, 8192), (40, 1024, 512)])
+def test_matmul_f8_scaled_parity_real_scales(m, k, n):
+    # random e4m3 codes and real-valued block scales against the oracle, tolerance 3e-2 (fp32 sums in another order)
+    announce('matmul_f8_scaled real scales', m, k, n)
+    rng = np.random.default_rng(m + k)
+    ac = O.e4m3_encode(rng.standard_normal((m, k)).astype(np.float32))
+    bc = O.e4m3_encode((rng.standard_normal((n, k)) * 0.5).astype(np.float32))
+    sa = rng.uniform(0.5, 2.0, (k // 128, m)).astype(np.float32)
+    sb = rng.uniform(0.01, 0.05, (n // 128, k // 128)).astype(np.float32)
+    got = F8.matmul_f8_scaled(f8(ac), f8(bc), scale_a=dev(sa), scale_b=dev(sb), output_dtype='float32')
+    ref = O.matmul_f8_scaled(ac, bc, sa, sb, 'float32')
+    err = O.max_rel_err(host(got), ref)
+    assert err <= 3e-2, err
+    assert err <= 1e-4, err  # fp32 accumulation on both sides: only the order of the sums differs
 
 
 @pytest.mark.parametrize('m,k,n', [(1, 8192, 8192), (16, 1024, 512), (256, 512, 768), (4096, 8192, 8192), (33, 400, 260)])
