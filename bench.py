@@ -312,7 +312,14 @@ def main():
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', al, wl[r % 3], sl, cl, 1, 8192, 28672, 8192, 0,
                                       work, work.numel(), sptr), 24, 6)
     others['w8a16_gemv_k8192_n28672_not_a_baseline_config'] = hbm_entry(us, 8192 * 28672 + 2 * 28672 + 2 * 8192 + 2 * 28672)
+    # what a kernel that only reads gets out of the memory system at these two sizes (16-byte loads, 32 KiB contiguous per
+    # workgroup, nothing else): the practical ceiling of the decode kernels, next to the data sheet's 8 TB/s
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    us = time_kernel(lambda r: ffi.call('hidet_qmm_read_probe', wl[r % 3], 8192 * 28672, sink, sptr), 24, 6)
+    read_probe = {'read_only_kernel_235MB': hbm_entry(us, 8192 * 28672)}
     del wl
+    us = time_kernel(lambda r: ffi.call('hidet_qmm_read_probe', ws[r % RING], K * N, sink, sptr), 64, 16)
+    read_probe['read_only_kernel_45MB'] = hbm_entry(us, K * N)
     # W8A16 prefill, attention QKV shape [2048, 4096] x [4096, 12288]
     wq = [torch.randint(-127, 128, (K, 12288), device=device, dtype=torch.int8) for _ in range(4)]
     sq = torch.cat([ss[0], ss[1]])[:12288].contiguous()
@@ -395,6 +402,7 @@ def main():
                                      'unit': 'TFLOP/s', 'frac': round(fp8_tflops / MFMA_FP8_PEAK_TFLOPS, 4)},
                         'max_rel_err_vs_oracle_rows_sample': fp8_parity, 'tolerance': 3e-2},
         'other_configs': others,
+        'read_probe': read_probe,
         'parity': {'max_rel_err_vs_oracle': parity, 'tolerance': 1e-2, 'graph_replay_matches_eager': replay_ok},
     }
     if not args.no_cpu_baseline:

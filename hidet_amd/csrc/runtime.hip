@@ -78,3 +78,29 @@ HIDET_API void hidet_qmm_arm_timing(void *start_event, void *stop_event) {
     ts.start = static_cast<hipEvent_t>(start_event);
     ts.stop = static_cast<hipEvent_t>(stop_event);
 }
+
+// ---- measurement: what a kernel that only reads can get out of the memory system -----------------------------------
+namespace {
+constexpr int kProbeBlockBytes = 32768;  // 256 threads x 8 loads x 16 bytes, contiguous per workgroup
+
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict__ src, uint32_t *__restrict__ sink) {
+    const uint4 *p = src + int64_t(blockIdx.x) * (kProbeBlockBytes / 16) + threadIdx.x;
+    uint4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = p[j * 256];
+    uint32_t acc = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    if (acc == 0x9E3779B9u) sink[0] = acc;  // practically never true; keeps the loads alive
+}
+}  // namespace
+
+HIDET_API void hidet_qmm_read_probe(const void *src, int64_t bytes, void *sink, void *stream) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(src && sink && qmm::aligned(src, 16), "null or misaligned pointer");
+    QMM_CHECK(bytes > 0 && bytes % kProbeBlockBytes == 0 && bytes / kProbeBlockBytes < (int64_t(1) << 31),
+              "the size must be a positive multiple of " << kProbeBlockBytes << " bytes, got " << bytes);
+    qmm::launch(read_probe_kernel, dim3(uint32_t(bytes / kProbeBlockBytes)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                static_cast<const uint4 *>(src), static_cast<uint32_t *>(sink));
+    QMM_ENTRY_END
+}

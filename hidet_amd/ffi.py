@@ -37,6 +37,7 @@ SIGNATURES = {
     'hidet_qmm_event_synchronize': (None, [_vp]),
     'hidet_qmm_event_elapsed_ms': (_f32, [_vp, _vp]),
     'hidet_qmm_arm_timing': (None, [_vp, _vp]),
+    'hidet_qmm_read_probe': (None, [_vp, _i64, _vp, _vp]),
     'hidet_symmetric_quantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _i64, _vp]),
     'hidet_symmetric_dequantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     'hidet_symmetric_quant_matmul_f16_i8': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),

@@ -63,6 +63,11 @@ void hidet_qmm_event_record(void *event, void *stream);
 void hidet_qmm_event_synchronize(void *event);
 float hidet_qmm_event_elapsed_ms(void *start, void *stop);
 void hidet_qmm_arm_timing(void *start_event, void *stop_event);
+/* Measurement only: one kernel that reads `bytes` (a multiple of 32768) from src with 16-byte loads, 32 KiB contiguous
+ * per workgroup, and does nothing else (sink: 4 bytes of device memory, practically never written).  Timed through the
+ * hook above it gives the rate at which this memory system delivers a matrix of that size to a kernel: the ceiling of
+ * the decode kernels at their real sizes, next to the 8 TB/s of the data sheet.  No counterpart in the reference. */
+void hidet_qmm_read_probe(const void *src, int64_t bytes, void *sink, void *stream);
 
 /* ---- symmetric quantize / dequantize ---------------------------------------------------------
  * replaces the auto-scheduled kernels of SymmetricQuantizationTask / SymmetricDeQuantizationTask
