@@ -4,7 +4,7 @@
 // rows per pass.
 //
 // The reduction runs along the contiguous axis, so nothing has to be exchanged between workgroups: a workgroup owns 16
-// output columns, its 4 waves split K and meet in LDS, N / 16 workgroups stream the weights exactly once.  Lane
+// output columns, its 4 or 8 waves split K and meet in LDS, N / 16 workgroups stream the weights exactly once.  Lane
 // (kg, ls) of a wave reads 32 consecutive bytes of row n0 + ls at k = kbase + 32 kg per 128-deep step (the 16 lanes x 4
 // k-groups of a step cover 16 rows x 128 contiguous bytes).  Bytes 8j .. 8j+7 of those 32 are, for j = 0 .. 3, the B
 // operand of one v_mfma_f32_16x16x32_f16: the k positions an MFMA sums over may be any 32 as long as both operands
@@ -13,12 +13,14 @@
 // (q ^ 0x80) == 1152 + q): one VALU op per weight; the constant is removed at the end with 1152 * sum_k a[m, k], which
 // one more MFMA per fragment (against ones) accumulates on the otherwise idle matrix pipe - exact in fp32 for the
 // few thousand terms of a wave's K range.  With K a multiple of 128 (FULL) the loop has no conditions at all: lanes
-// of rows >= M and columns >= N read a clamped row and their results are dropped at the end.
+// of rows >= M and columns >= N read a clamped row and their results are dropped at the end.  Each step of that loop
+// sits behind a wave-uniform break, and the compiler moves the step's loads down into its block: a wave has one step in
+// flight at a time and the 8 to 11 waves per CU hide the latency (the FP8 kernel of the same shape was measured a third
+// slower with all of a trip's loads really issued up front).
 #include "common.h"
 
 namespace qmm {
 namespace {
-
 
 template <bool ALIGNED_A, bool FULL, int WAVES, bool STAGE = false>
 __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Float16 *__restrict__ a, int64_t lda,
@@ -26,7 +28,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
                                                               const _Float16 *__restrict__ scale, _Float16 *__restrict__ c,
                                                               int m, int k, int n) {
     __shared__ float red[WAVES][16][17];
-    constexpr int kNkDepth = FULL ? 8 : 4;  // 128-deep steps whose loads are issued together
+    constexpr int kNkDepth = FULL ? 8 : 4;  // 128-deep steps per trip of the outer loop
     // STAGE (FULL with aligned activations, more than two rows): a wave fetches its 16 x 128 activation block of a step
     // with four fully coalesced loads (4 rows x 256 bytes each) and turns it into MFMA fragments through a private LDS
     // tile of 16 rows x (256 + 16) bytes, two slots.  Fetching the fragments straight from memory touches every cache
