@@ -61,15 +61,15 @@ _ROW_MAJOR_COPIES = WeakTensorKeyDictionary()  # K-contiguous weight tensor (by 
 
 def _row_major(weight: torch.Tensor) -> torch.Tensor:
     """`weight` as the row-major [K, N] tensor the GEMM and the N-contiguous GEMV read.  The copy of a K-contiguous weight
-    (45 MB for a 4096 x 11008 layer) is made once per tensor object and lives as long as that object does; a weight that
-    is modified in place afterwards must be passed as a new tensor."""
+    (45 MB for a 4096 x 11008 layer) is made once per tensor object and lives as long as that object does; it is made again
+    when the weight has been written in place since (torch's version counter)."""
     if weight.is_contiguous():
         return weight
     if weight.dim() == 2 and weight.stride(0) == 1:
-        copy = _ROW_MAJOR_COPIES.get(weight)
-        if copy is None or copy.device != weight.device:
-            copy = _ROW_MAJOR_COPIES[weight] = weight.contiguous()
-        return copy
+        entry = _ROW_MAJOR_COPIES.get(weight)
+        if entry is None or entry[0] != weight._version or entry[1].device != weight.device:
+            entry = _ROW_MAJOR_COPIES[weight] = (weight._version, weight.contiguous())
+        return entry[1]
     return weight.contiguous()
 
 

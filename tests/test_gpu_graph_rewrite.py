@@ -149,4 +149,11 @@ def test_decode_layout_runs_decode_and_prefill_calls():
         assert got.shape == want.shape
         assert O.max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) < 2e-3
     from hidet_amd.graph.ops.quant import matmul as qmm
-    assert qmm._ROW_MAJOR_COPIES.get(gm.up_weight_wq_kc) is not None
+    entry = qmm._ROW_MAJOR_COPIES.get(gm.up_weight_wq_kc)
+    assert entry is not None and entry[1].is_contiguous() and torch.equal(entry[1], gm.up_weight_wq_kc)
+    # a weight written in place gets a fresh copy on the next prefill-sized call
+    gm.up_weight_wq_kc.zero_()
+    x = torch.randn(40, 512, device='cuda', dtype=torch.float16)
+    with torch.no_grad():
+        gm(x)
+    assert int(qmm._ROW_MAJOR_COPIES.get(gm.up_weight_wq_kc)[1].abs().sum()) == 0
