@@ -36,7 +36,10 @@ def test_quantize_per_tensor_bit_exact():
     c0, s0 = O.fp8_quantize_per_tensor(x)
     assert float(scale.item()) == 1.0 == float(s0)
     assert np.array_equal(codes_of(codes), c0)
-    for shape, dt in (((300, 70), torch.float32), ((64, 64), torch.bfloat16), ((1, 5), torch.float16), ((0,), torch.float32)):
+    for shape, dt in (((300, 70), torch.float32), ((64, 64), torch.bfloat16), ((1, 5), torch.float16), ((0,), torch.float32),
+                      # more than 65536 elements: the two-pass kernels; 16-bit inputs with and without whole 16-byte groups
+                      ((400, 200), torch.float32), ((513, 136), torch.float16), ((513, 136), torch.bfloat16),
+                      ((257, 260), torch.bfloat16), ((2100, 1024), torch.bfloat16)):
         y = (rng.standard_normal(shape) * 3).astype(np.float32)
         ty = dev(y).to(dt)
         y = ty.float().cpu().numpy()
