@@ -687,7 +687,7 @@ HIDET_API void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *s
             return;
         }
         if (numel > 0) {
-            const int64_t blocks = std::min<int64_t>(cdiv(numel, 256 * 8), 2048);
+            const int64_t blocks = std::min<int64_t>(cdiv(numel, 256 * 8), 512);  // one atomic on one word per workgroup
             launch(amax_all_kernel<DT>, dim3(blocks), dim3(256), 0, stream, x, amax_bits, numel);
         }
         launch(fp8_quantize_kernel<DT>, dim3(std::max<int64_t>(1, cdiv(numel, 256))), dim3(256), 0, stream, x, amax_bits,
