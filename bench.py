@@ -386,8 +386,14 @@ def main():
     c1 = torch.empty((1, NF), dtype=torch.bfloat16, device=device)
     bring = [bq for bq, _ in b8s] + [torch.randint(0, 0x7F, (NF, KF), device=device, dtype=torch.uint8) for _ in range(5)]  # 8 x 64 MiB
     us = time_kernel(lambda r: ffi.call('hidet_matmul_f8', a1, bring[r % 8], c1, 1, NF, KF, KF, KF, 2, sa, b8s[0][1], work, work.numel(), sptr), 32, 8)
-    del bring
     others['fp8_gemv_m1_k8192_n8192'] = hbm_entry(us, NF * KF + KF + 2 * NF + 8)
+    # the block-scaled form of the same GEMV (scale_a f32 [K/128, 1], scale_b f32 [N/128, K/128])
+    bsa = torch.rand((KF // 128, 1), generator=g, device=device, dtype=torch.float32) + 0.5
+    bsb = torch.rand((NF // 128, KF // 128), generator=g, device=device, dtype=torch.float32) + 0.5
+    us = time_kernel(lambda r: ffi.call('hidet_matmul_f8_scaled', a1, bring[r % 8], bsa, bsb, c1, 1, NF, KF, 2, work, work.numel(),
+                                      sptr), 32, 8)
+    others['fp8_block_scaled_gemv_m1_k8192_n8192'] = hbm_entry(us, NF * KF + KF + 2 * NF + 4 * (KF // 128) * (1 + NF // 128))
+    del bring
 
     if args.data_dependence:
         def timed(fn, reps=24):
