@@ -207,7 +207,7 @@ def test_gemm_k_split_matches_unsplit_and_is_deterministic():
 @pytest.mark.parametrize('m,k,n', [(1, 4096, 11008), (1, 11008, 4096), (16, 4096, 4096), (3, 512, 48), (7, 144, 20), (1, 16, 2),
                                    (20, 1024, 264), (32, 4096, 512), (2, 384, 32), (5, 1152, 8200), (4, 2176, 8192),
                                    (9, 1040, 40), (9, 1152, 8200), (16, 4096, 11008), (5, 1024, 8192), (21, 1280, 8256), (12, 8192, 8200), (3, 2048, 64),
-                                   (16, 1024, 8192)])
+                                   (16, 1024, 8192), (2, 16384, 48), (3, 32768, 16)])
 def test_k_contiguous_weights_exact(m, k, n):
     # the [K, N] weight held with strides (1, K): same operator, same results, the kernel that reduces along the
     # contiguous axis; small integers make every product and partial sum exact.  K a multiple of 128 or not, 4 and 8
