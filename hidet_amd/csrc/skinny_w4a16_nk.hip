@@ -151,8 +151,12 @@ void skinny_w4a16_nk_launch(const void *a, const void *w, const void *scales, vo
         // or two rows they also shorten each wave's chain of dependent steps (K = 4096, N = 11008, one row: 9.6 -> 9.1 us;
         // 4 to 16 rows: 9.8-11.2 -> 10.5-11.5 us, so not there)
         const bool eight = (cdiv(n, 16) < 512 || !stage) && k >= 8 * 128;
+        // few column tiles, a long K and one or two rows: sixteen waves halve each wave's chain of steps once more
+        // (K = 11008, N = 4096: 10.5 -> 8.7 us; with the LDS tile of the staged form 16 waves would not fit)
+        const bool sixteen = cdiv(n, 16) < 512 && !stage && k >= 32 * 128;
 #define QMM_W4_NK(DT)                                                                \
-    if (eight && stage) go(skinny_w4a16_nk_kernel<DT, 8, true>, 8);                  \
+    if (sixteen) go(skinny_w4a16_nk_kernel<DT, 16, false>, 16);                      \
+    else if (eight && stage) go(skinny_w4a16_nk_kernel<DT, 8, true>, 8);             \
     else if (eight) go(skinny_w4a16_nk_kernel<DT, 8, false>, 8);                     \
     else if (stage) go(skinny_w4a16_nk_kernel<DT, 4, true>, 4);                      \
     else go(skinny_w4a16_nk_kernel<DT, 4, false>, 4);

@@ -90,7 +90,8 @@ def test_exact_on_small_integers():
 
 
 @pytest.mark.parametrize('m,k,n,g', [(1, 4096, 11008, 128), (16, 4096, 11008, 128), (2, 1024, 4096, 256), (5, 384, 40, 128),
-                                     (9, 1152, 72, 128), (3, 128, 16, 128), (21, 2048, 528, 1024), (1, 11008 - 11008 % 128, 4096, 128)])
+                                     (9, 1152, 72, 128), (3, 128, 16, 128), (21, 2048, 528, 1024), (1, 11008 - 11008 % 128, 4096, 128),
+                                     (2, 4096, 4096, 128)])  # the last two: sixteen waves per workgroup
 @pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
 def test_decode_layout_parity_and_same_result_as_row_major(m, k, n, g, dtype):
     # the weight repacked K-contiguous for decode: same operator, compared with the oracle and with the row-major kernels
