@@ -122,7 +122,7 @@ def main():
             c_nk = torch.empty((1, N), dtype=torch.float16, device=device)
             for rep in range(2):
                 for i in range(RING):
-                    ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a, ws[i].view(N, K), ss[0], c_nk, 1, K, N, K, K, sptr)
+                    ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a, ws[i].view(N, K), ss[0], c_nk, 1, K, N, K, K, None, 0, sptr)
         stream.synchronize()
         print(json.dumps({'pmc_calibration': {'copy_bytes': 64 << 20, 'copies': 4, 'gemv_launches': 2 * RING,
                                               'gemv_k_contiguous_launches': 2 * RING, 'gemv_algorithmic_bytes': GEMV_BYTES}}))
@@ -321,7 +321,7 @@ def main():
                                       work, work.numel(), sptr), 96, 32)
     others['w8a16_m16_k4096_n4096'] = hbm_entry(us, 4096 * 4096 + 2 * 4096 + 2 * 16 * 4096 * 2)
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a16, w16[r % 32], s16, c16, 16, 4096, 4096, 4096, 4096,
-                                      sptr), 96, 32)  # the same buffers read as [N, K] storage
+                                      None, 0, sptr), 96, 32)  # the same buffers read as [N, K] storage
     others['w8a16_m16_k4096_n4096_k_contiguous_weights'] = hbm_entry(us, 4096 * 4096 + 2 * 4096 + 2 * 16 * 4096 * 2)
     del w16
     # W8A16 decode GEMV, down-proj shape [1, 11008] x [11008, 4096]: the ring's buffers reinterpreted as [11008, 4096]
@@ -335,10 +335,10 @@ def main():
     # another data layout than the benchmark configuration's, so never the headline; the ring's buffers reinterpreted
     cu = torch.empty((1, N), dtype=torch.float16, device=device)
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a, ws[r % RING].view(N, K), ss[0], cu, 1, K, N, K, K,
-                                      sptr), 48, 16)
+                                      None, 0, sptr), 48, 16)
     others['w8a16_gemv_k4096_n11008_k_contiguous_weights'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * N)
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ad, ws[r % RING].view(K, N), sd, cd, 1, N, K, N, N,
-                                      sptr), 48, 16)
+                                      None, 0, sptr), 48, 16)
     others['w8a16_gemv_down_proj_k11008_n4096_k_contiguous_weights'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * K)
     # the same GEMV kernel on a matrix five times the size (not a benchmark configuration: it shows how much of the headline
     # figure is the fixed cost of one launch and one cross-workgroup exchange)

@@ -10,6 +10,10 @@ void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c,
 bool skinny_w8a16_nk_supported(const void *w, int64_t k, int64_t ldw);
 void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                             int64_t lda, int64_t ldw, hipStream_t stream);
+bool gemm_w8a16_nk_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                             int64_t ldw);
+void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
+                          int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 }
 
 using namespace qmm;
@@ -40,17 +44,26 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
 }
 
 HIDET_API void hidet_symmetric_quant_matmul_f16_i8_nk(const void *a, const void *w_nk, const void *scale, void *c, int64_t m,
-                                                      int64_t k, int64_t n, int64_t lda, int64_t ldw, void *stream_) {
+                                                      int64_t k, int64_t n, int64_t lda, int64_t ldw, void *workspace,
+                                                      int64_t workspace_bytes, void *stream_) {
     QMM_ENTRY_BEGIN
     QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
     QMM_CHECK(lda >= k && ldw >= k, "row strides (" << lda << ", " << ldw << ") must be at least K (" << k << ")");
     QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    QMM_CHECK(workspace_bytes >= 0 && (workspace == nullptr || aligned(workspace, 16)),
+              "the workspace must be 16-byte aligned (or NULL: no tile is computed in K ranges)");
     if (m == 0 || n == 0) return;
     QMM_CHECK(a && w_nk && scale && c, "null tensor pointer");
     QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
     QMM_CHECK(skinny_w8a16_nk_supported(w_nk, k, ldw),
               "K-contiguous weights need K and the row stride to be multiples of 16 and a 16-byte aligned pointer, got K=" << k
                                                                                                                          << " ldw=" << ldw);
-    skinny_w8a16_nk_launch(a, w_nk, scale, c, m, k, n, lda, ldw, static_cast<hipStream_t>(stream_));
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    // more than one pass of 16 rows: the MFMA GEMM reading the same layout, where its conditions hold
+    if (m > 16 && gemm_w8a16_nk_supported(a, w_nk, c, m, k, n, lda, ldw))
+        gemm_w8a16_nk_launch(a, w_nk, scale, c, m, k, n, lda, ldw, workspace ? workspace : nullptr,
+                             workspace ? workspace_bytes : 0, stream);
+    else
+        skinny_w8a16_nk_launch(a, w_nk, scale, c, m, k, n, lda, ldw, stream);
     QMM_ENTRY_END
 }

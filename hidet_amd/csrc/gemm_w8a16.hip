@@ -41,9 +41,11 @@ struct GemmW8Cfg16 {
 
 // RBA <= RB: row blocks (of 16 rows) per wave that can hold rows of the matrix. A short matrix (M <= 16 RBA) runs the same
 // tile with the activation loads, fragment reads and MFMAs of the other row blocks left out.
-template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA>
+// W_NK: the weight is stored K-contiguous, w[col * ldw + k] (the [N, K] storage of nn.Linear); a lane then loads the 8
+// consecutive k of one of its 4 columns with one 8-byte load and widens byte pairs instead of gathering rows.
+template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA, bool W_NK = false>
 __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(const _Float16 *__restrict__ a, int64_t lda,
-                                                                                 const int8_t *__restrict__ w,
+                                                                                 const int8_t *__restrict__ w, int64_t ldw,
                                                                                  const _Float16 *__restrict__ scale,
                                                                                  _Float16 *__restrict__ c, int m, int k, int n,
                                                                                  int tiles_m, int tiles_n, int xm, int xn,
@@ -73,8 +75,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[rb][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const __amdgpu_buffer_rsrc_t rsrc_w =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(w), 0, int(int64_t(k) * n), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t *>(w), 0, W_NK ? int(int64_t(n - 1) * ldw + k) : int(int64_t(k) * n), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<_Float16 *>(a), 0, int((int64_t(m - 1) * lda + k) * 2), 0x00020000);
 
@@ -89,9 +91,13 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         const int row = m0 + r;
         a_off[j] = row < m ? int((int64_t(row) * lda + ((id & 7) ^ lds_swizzle_key_step1(r)) * 8) * 2) : 0x7FFFFFF0;
     }
-    int w_off[8];
+    // row-major: row 8 kg + j of a k-step, 4 columns; K-contiguous: column col + t, the 8 k of lane group kg
+    int w_off[W_NK ? 4 : 8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w_off[j] = col_ok ? (kg * 8 + j) * n + col : 0x7FFFFFF0;
+    for (int j = 0; j < (W_NK ? 4 : 8); ++j)
+        w_off[j] = !col_ok ? 0x7FFFFFF0 : W_NK ? int(int64_t(col + j) * ldw) + kg * 8 : (kg * 8 + j) * n + col;
+    constexpr int kWLoadsPerStage = W_NK ? 8 : 16;  // weight load instructions of one stage
+    constexpr uint32_t kPairLo = 0x0c010c00u, kPairHi = 0x0c030c02u;  // bytes (0, 1) / (2, 3) of a dword into two halves
 
     const int stages = k / kBK;
     const int s_begin = (stages * part) / parts, s_end = (stages * (part + 1)) / parts;
@@ -114,11 +120,32 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
                                     (st < stages ? st : stages - 1) * (kBK * 2));  // the scalar offset is not range-checked
     };
     auto load_w = [&](int st, int q, uint32_t (&dst)[8]) {
-        const int soff = ((st < stages ? st : stages - 1) * kBK + q * 32) * n;
+        if constexpr (W_NK) {
+            const int soff = (st < stages ? st : stages - 1) * kBK + q * 32;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dst[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[j], soff, 0);
+            for (int t = 0; t < 4; ++t) {
+                const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_off[t], soff, 0);
+                dst[2 * t] = v[0];
+                dst[2 * t + 1] = v[1];
+            }
+        } else {
+            const int soff = ((st < stages ? st : stages - 1) * kBK + q * 32) * n;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_w, w_off[j], soff, 0);
+        }
     };
     auto dequant = [&](const uint32_t (&raw)[8], BFrag (&dst)[4]) {
+        if constexpr (W_NK) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const uint32_t src = raw[2 * t + p / 2];
+                    dst[t].u[p] = __builtin_amdgcn_perm(src, src, (p & 1) ? kPairHi : kPairLo) ^ 0x64806480u;
+                    dst[t].h2[p] = dst[t].h2[p] - half2_t{_Float16(1152.0f), _Float16(1152.0f)};
+                }
+            return;
+        }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             constexpr uint32_t kZero = 0x0c;
@@ -160,7 +187,24 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
             constexpr int Q = IDX / RB, RBI = IDX % RB;
             constexpr int AI = Q * RBA + RBI;  // fragment index, if the row block is active
             if constexpr (RBI < RBA) issue(std::integral_constant<int, AI + 3>());
-            {
+            if constexpr (W_NK) {
+                constexpr int T = RBI / 2;  // column of the next k-step's block; this block widens one of its two dwords
+                const uint32_t src = w_raw[Q ^ 1][2 * T + (RBI & 1)];
+                BFrag &dst = bq[Q ^ 1][T];
+#pragma unroll
+                for (int pp = 0; pp < 2; ++pp) {
+                    constexpr int kFirst = 2 * (RBI & 1);
+                    dst.u[kFirst + pp] = __builtin_amdgcn_perm(src, src, pp ? kPairHi : kPairLo) ^ 0x64806480u;
+                    dst.h2[kFirst + pp] = dst.h2[kFirst + pp] - half2_t{_Float16(1152.0f), _Float16(1152.0f)};
+                }
+                if constexpr (RBI & 1) {  // both dwords of column T are consumed: refill them one stage ahead
+                    const int st = Q == 0 ? s + 1 : s + 2;
+                    const int soff = (st < stages ? st : stages - 1) * kBK + (Q ^ 1) * 32;
+                    const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_off[T], soff, 0);
+                    w_raw[Q ^ 1][2 * T] = v[0];
+                    w_raw[Q ^ 1][2 * T + 1] = v[1];
+                }
+            } else {
                 constexpr int P = RBI / 2;  // row pair of the next k-step's raw block
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
@@ -205,8 +249,8 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         kstep(std::integral_constant<int, 0>());
         kstep(std::integral_constant<int, 1>());
         // the loads of stage s + 1 (issued one stage ago) must have landed in LDS before anyone reads them; the
-        // loads issued during this stage (kAChunksActive + 16 of them) may stay in flight
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(kAChunksActive + 16));
+        // loads issued during this stage (kAChunksActive + kWLoadsPerStage of them) may stay in flight
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(kAChunksActive + kWLoadsPerStage));
         __syncthreads();
     };
 
@@ -256,9 +300,9 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
         }
 }
 
-template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA>
+template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA, bool W_NK = false>
 void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
-                  void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+                  int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     using Cfg = GemmW8Cfg16<RB, WM, WN>;
     const int tiles_m = int(cdiv(m, Cfg::kBM)), tiles_n = int(cdiv(n, Cfg::kBN));
     constexpr int kConcurrent = 32 * MIN_BLOCKS;  // workgroups an XCD (32 CUs) runs at a time
@@ -283,9 +327,9 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     static_assert(8 * kConcurrent * 4 <= kCounterBytes, "one counter per tail tile");
     const int64_t grid = gemm_grid_with_tail(tiling, split_unit, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>), Cfg::kLdsBytes);
-    launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
-           static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale),
+    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA, W_NK>), Cfg::kLdsBytes);
+    launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA, W_NK>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
+           static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale),
            static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, split_unit, tail.parts, tail.max_tiles,
            reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
 }
@@ -302,10 +346,26 @@ bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     // waves 128 x 64, workgroup tile 128 x 256; a matrix of at most 32 / 64 / 96 rows leaves the empty row blocks out
-    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
-    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
-    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
-    else launch_cfg16<8, 1, 4, 2, 8>(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
+    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    else launch_cfg16<8, 1, 4, 2, 8>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+}
+
+// The same kernel on a weight stored K-contiguous (w_nk[col * ldw + k]): 8-byte loads, so rows of w_nk 8-byte aligned.
+bool gemm_w8a16_nk_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                             int64_t ldw) {
+    return (k % kBK == 0) && (lda % 8 == 0) && (n % 4 == 0) && (ldw % 8 == 0) && aligned(a, 16) && aligned(w, 8) &&
+           aligned(c, 8) && (n - 1) * ldw + k < (int64_t(1) << 31) - (1 << 20) &&
+           (m * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
+}
+
+void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
+                          int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+    else launch_cfg16<8, 1, 4, 2, 8, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
 }
 
 }  // namespace qmm

@@ -40,16 +40,22 @@ class SymmetricQuantizedMatmulTask(Task):
                          outputs=[TensorSpec('c', 'float16', c_shape)], attrs={})
 
 
-_NK_MAX_ROWS = 16  # one pass of the K-contiguous kernel; more rows are served better by the MFMA GEMM on row-major codes
+_NK_MAX_ROWS = 16  # one pass of the bandwidth-bound kernels for K-contiguous weights; more rows go to the MFMA GEMM
+# The GEMM that reads K-contiguous weights gathers 8 bytes per lane from 16 rows of the stored matrix per load and runs
+# about a third slower than the row-major one at prefill sizes (2048 x 4096 x 11008: 214 against 157 us; 64 rows: 25 against
+# 20 us).  Batched decode (17 to 64 rows) uses it, so a model that only decodes never makes a second copy of its weights;
+# longer prompts use the row-major copy.
+_NK_GEMM_MAX_ROWS = 64
 
 
 def to_decode_layout(wq: torch.Tensor) -> torch.Tensor:
     """The same [K, N] int8 weight, stored K-contiguous (a view with strides (1, K) of a fresh [N, K] tensor).
 
     `symmetric_quant_matmul` on such a weight with up to 16 activation rows runs the kernel that
-    reduces along the contiguous axis (no exchange between workgroups); it is what `nn.Linear` stores, so `linear.weight`
-    quantized with `dims=1` and viewed with `.t()` is already in this layout.  A call with more rows makes a row-major copy
-    of the weight the first time and keeps it for as long as the weight tensor lives.
+    reduces along the contiguous axis (no exchange between workgroups), with up to 64 the MFMA GEMM that reads this layout;
+    it is what `nn.Linear` stores, so `linear.weight` quantized with `dims=1` and viewed with `.t()` is already in this
+    layout.  A call with more rows makes a row-major copy of the weight the first time and keeps it for as long as the
+    weight tensor lives.
     """
     if wq.dim() != 2:
         raise ValueError('expected a 2-D weight, got shape {}'.format(list(wq.shape)))
@@ -85,12 +91,16 @@ def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parall
     lda = a2.stride(0) if m > 1 else k
     scale = scale.contiguous()
     c = torch.empty((m, n), dtype=torch.float16, device=a.device)
-    # A [K, N] weight held K-contiguous (strides (1, ldw): `wq_nk.t()` of an [N, K] tensor, see `to_decode_layout`) goes to the
-    # kernel that reduces along the contiguous axis when the call is a decode-sized one; otherwise it is copied to the
-    # row-major layout the other kernels read, as any non-contiguous operand is.
-    if (m <= _NK_MAX_ROWS and k > 1 and n > 1 and weight.stride(0) == 1 and weight.stride(1) >= k and weight.stride(1) % 16 == 0
-            and k % 16 == 0 and weight.data_ptr() % 16 == 0):
-        ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a2, weight, scale, c, m, k, n, lda, weight.stride(1),
+    # A [K, N] weight held K-contiguous (strides (1, ldw): `wq_nk.t()` of an [N, K] tensor, see `to_decode_layout`) goes to
+    # the entry point for that layout: the bandwidth-bound kernels up to 16 rows, the MFMA GEMM reading the same layout up
+    # to 64 (K a multiple of 64, N of 4).  What neither takes uses a row-major copy, as any non-contiguous operand does.
+    if (k > 1 and n > 1 and weight.stride(0) == 1 and weight.stride(1) >= k and weight.stride(1) % 16 == 0
+            and k % 16 == 0 and weight.data_ptr() % 16 == 0
+            and (m <= _NK_MAX_ROWS or (m <= _NK_GEMM_MAX_ROWS and k % 64 == 0 and n % 4 == 0 and lda % 8 == 0 and a2.data_ptr() % 16 == 0
+                                       and (n - 1) * weight.stride(1) + k < (1 << 31) - (1 << 20)
+                                       and (m * lda + k) * 2 < (1 << 31) - (1 << 20)))):
+        ws = ffi.workspace(a.device)
+        ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a2, weight, scale, c, m, k, n, lda, weight.stride(1), ws, ws.numel(),
                  ffi.current_stream(a.device))
         return c.reshape(tuple(a.shape[:-1]) + (n,))
     weight = _row_major(weight)

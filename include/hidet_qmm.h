@@ -96,10 +96,12 @@ void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const voi
  * python/hidet/graph/ops/matmul/matmul.py:37-38, python/hidet/graph/frontend/torch/register_functions.py:165-167).
  * The reference's quantized operator has no such form (its rewrite rule re-emits the matmul without transpose_b,
  * python/hidet/graph/transforms/graph_patterns/quant/linear.py:43-49).  The reduction then runs along the
- * contiguous axis and needs no workspace.  Meant for decode (a few rows): every 16 rows of a are one more pass over
- * the weights.  K and ldw multiples of 16, w_nk 16-byte aligned. */
+ * contiguous axis: up to 16 rows take the bandwidth-bound kernels, which need no workspace; more rows the MFMA GEMM
+ * reading this layout (K a multiple of 64; the workspace is optional, NULL means no tile is computed in K ranges,
+ * which matters below a few hundred rows).  K and ldw multiples of 16, w_nk 16-byte aligned. */
 void hidet_symmetric_quant_matmul_f16_i8_nk(const void *a, const void *w_nk, const void *scale, void *c, int64_t m,
-                                            int64_t k, int64_t n, int64_t lda, int64_t ldw, void *stream);
+                                            int64_t k, int64_t n, int64_t lda, int64_t ldw, void *workspace,
+                                            int64_t workspace_bytes, void *stream);
 
 /* ---- group-wise W4A16 (benchmark configuration; the reference has no operator for it) -----------
  * Conventions inherited from the reference: int4b is signed with max 7, so the symmetric rule of

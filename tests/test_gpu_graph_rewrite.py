@@ -142,7 +142,8 @@ def test_decode_layout_runs_decode_and_prefill_calls():
         ctx.set_precision('int8').set_decode_layout()
         gm = quantize_module(model, ctx)
     assert gm.up_weight_wq_kc.stride() == (1, 512) and torch.equal(gm.up_weight_wq_kc, plain.up_weight_wq)
-    for rows in (1, 3, 40, 16, 1):  # decode-sized calls, a prefill-sized one (row-major copy made once), decode again
+    for rows in (1, 3, 40, 100, 16, 1):  # decode-sized calls, batched decode (the GEMM on the same layout), a prefill-sized one
+                                         # (row-major copy made once), decode again
         x = torch.randn(rows, 512, device='cuda', dtype=torch.float16)
         with torch.no_grad():
             got, want = gm(x), plain(x)
@@ -153,7 +154,7 @@ def test_decode_layout_runs_decode_and_prefill_calls():
     assert entry is not None and entry[1].is_contiguous() and torch.equal(entry[1], gm.up_weight_wq_kc)
     # a weight written in place gets a fresh copy on the next prefill-sized call
     gm.up_weight_wq_kc.zero_()
-    x = torch.randn(40, 512, device='cuda', dtype=torch.float16)
+    x = torch.randn(100, 512, device='cuda', dtype=torch.float16)
     with torch.no_grad():
         gm(x)
     assert int(qmm._ROW_MAJOR_COPIES.get(gm.up_weight_wq_kc)[1].abs().sum()) == 0

@@ -207,7 +207,10 @@ def test_gemm_k_split_matches_unsplit_and_is_deterministic():
 @pytest.mark.parametrize('m,k,n', [(1, 4096, 11008), (1, 11008, 4096), (16, 4096, 4096), (3, 512, 48), (7, 144, 20), (1, 16, 2),
                                    (20, 1024, 264), (32, 4096, 512), (2, 384, 32), (5, 1152, 8200), (4, 2176, 8192),
                                    (9, 1040, 40), (9, 1152, 8200), (16, 4096, 11008), (5, 1024, 8192), (21, 1280, 8256), (12, 8192, 8200), (3, 2048, 64),
-                                   (16, 1024, 8192), (2, 16384, 48), (3, 32768, 16)])
+                                   (16, 1024, 8192), (2, 16384, 48), (3, 32768, 16),
+                                   # more than 16 rows: the MFMA GEMM on the same layout (row blocks left out, K ranges, ragged edges)
+                                   (17, 4096, 11008), (100, 512, 264), (129, 4096, 512), (300, 256, 1056), (520, 2048, 264),
+                                   (33, 4096, 520), (700, 1024, 2048), (64, 192, 8), (40, 1040, 64)])
 def test_k_contiguous_weights_exact(m, k, n):
     # the [K, N] weight held with strides (1, K): same operator, same results, the kernel that reduces along the
     # contiguous axis; small integers make every product and partial sum exact.  K a multiple of 128 or not, 4 and 8
@@ -224,7 +227,8 @@ def test_k_contiguous_weights_exact(m, k, n):
     assert np.array_equal(host(quant.symmetric_quant_matmul(ta, w_nk, ts)), want)
     # the entry point itself, whatever the row count
     c = torch.full((m, n), float('nan'), dtype=torch.float16, device='cuda')
-    hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ta, w_nk, ts, c, m, k, n, k, k,
+    ws = hidet_amd.ffi.workspace(c.device)
+    hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ta, w_nk, ts, c, m, k, n, k, k, ws, ws.numel(),
                        hidet_amd.ffi.current_stream(c.device))
     assert np.array_equal(host(c), want)
 
@@ -261,4 +265,4 @@ def test_k_contiguous_weights_parity_and_fallback():
     with pytest.raises(hidet_amd.BackendException):
         ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', torch.zeros(1, 24, device='cuda', dtype=torch.float16), bad,
                  torch.zeros(8, device='cuda', dtype=torch.float16), torch.zeros(1, 8, device='cuda', dtype=torch.float16),
-                 1, 24, 8, 24, 24, ffi.current_stream(bad.device))
+                 1, 24, 8, 24, 24, None, 0, ffi.current_stream(bad.device))
