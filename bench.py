@@ -364,6 +364,16 @@ def main():
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ap, wq[r % 4], sq, cq, MP, K, 12288, K, 0, work,
                                       work.numel(), sptr), 16, 4)
     others['w8a16_prefill_m2048_k4096_n12288'] = mfma_entry(us, 2.0 * MP * K * 12288, MFMA_F16_PEAK_TFLOPS)
+    # the M = 2048 prefill GEMM on K-contiguous weights (the ring's buffers read as [N, K] storage; another layout), and 32 rows
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ap, ws[r % RING].view(N, K), ss[0], cp, MP, K, N, K, K,
+                                      work, work.numel(), sptr), 16, 4)
+    others['w8a16_prefill_m2048_k4096_n11008_k_contiguous_weights'] = mfma_entry(us, 2.0 * MP * K * N, MFMA_F16_PEAK_TFLOPS)
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ap[:32], ws[r % RING].view(N, K), ss[0], cp[:32], 32, K, N,
+                                      K, K, work, work.numel(), sptr), 32, 16)
+    others['w8a16_m32_k4096_n11008_k_contiguous_weights'] = hbm_entry(us, K * N + 2 * N + 2 * 32 * (K + N))
+    us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ap[:32], ws[r % RING], ss[0], cp[:32], 32, K, N, K, 0,
+                                      work, work.numel(), sptr), 32, 16)
+    others['w8a16_m32_k4096_n11008'] = hbm_entry(us, K * N + 2 * N + 2 * 32 * (K + N))
     del wq, cq
     # group-wise W4A16 (bf16, group 128), M in {1, 16, 512}
     w4 = [torch.randint(0, 256, (K, N // 2), device=device, dtype=torch.uint8) for _ in range(16)]
