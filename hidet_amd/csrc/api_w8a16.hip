@@ -3,7 +3,8 @@
 
 namespace qmm {
 void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace,
+                         hipStream_t stream);
 bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda);
 void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
                        int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream);
@@ -18,10 +19,12 @@ void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, void 
 
 using namespace qmm;
 
-HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
-                                                   int64_t k, int64_t n, int64_t lda, int parallel_k_parts,
-                                                   void *workspace, int64_t workspace_bytes, void *stream_) {
-    QMM_ENTRY_BEGIN
+namespace {
+
+// Checks and kernel choice shared by the two row-major entry points. `strict_workspace`: a bandwidth-bound launch whose
+// K split does not fit the scratch memory is an error instead of a launch with fewer K slices.
+void w8a16_dispatch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                    int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace, hipStream_t stream) {
     QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
     QMM_CHECK(lda >= k, "row stride of a (" << lda << ") is smaller than K (" << k << ")");
     QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
@@ -29,7 +32,6 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
     if (m == 0 || n == 0) return;
     QMM_CHECK(a && w && scale && c, "null tensor pointer");
     QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     // Up to 16 rows one pass of the bandwidth-bound kernel serves; beyond that every 16 rows would cost another pass
     // over the weights, and the MFMA GEMM with its K split and its empty row blocks left out takes over (K=4096, N=11008,
     // weights from HBM: 17 us at M=17..32, 20 us at M=64, 29 us at M=128). From 9 rows on the GEMM is already ahead when
@@ -39,7 +41,18 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
     if ((m > 16 || (m > 8 && wide && parallel_k_parts == 0)) && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
         gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
-        skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, stream);
+        skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, strict_workspace,
+                            stream);
+}
+
+}  // namespace
+
+HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
+                                                   int64_t k, int64_t n, int64_t lda, int parallel_k_parts,
+                                                   void *workspace, int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    w8a16_dispatch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, false,
+                   static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }
 

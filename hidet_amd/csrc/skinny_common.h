@@ -178,4 +178,26 @@ inline void skinny_plan(int64_t k, int64_t n, int slice_rows, int hint_parts, in
     *tiles = int(t);
 }
 
+// Bytes of workspace a skinny launch with `splits` K slices touches: the counters and one fp32 partial tile per
+// (column tile, K slice) of `rows` (at most 16) activation rows. One slice exchanges nothing.
+inline int64_t skinny_workspace_need(int tiles, int splits, int rows) {
+    return splits > 1 ? kCounterBytes + int64_t(tiles) * splits * rows * kSkinnyTileN * 4 : 0;
+}
+
+// Makes the plan fit the caller's workspace: fewer, longer K slices (down to one, which needs no workspace) when the
+// partial tiles would not fit. `strict` callers get an error instead, naming the bytes the plan needs.
+inline void skinny_fit_workspace(int64_t k, int granule, int tiles, int rows, const void *workspace, int64_t workspace_bytes,
+                                 bool strict, int *rows_per_block, int *splits) {
+    const int64_t avail = workspace != nullptr ? workspace_bytes : 0;
+    const int64_t need = skinny_workspace_need(tiles, *splits, rows);
+    if (need <= avail) return;
+    if (strict) QMM_FAIL("scratch too small for this shape: the K split needs " << need << " bytes, " << avail << " are there");
+    const int64_t per_split = int64_t(tiles) * rows * kSkinnyTileN * 4;
+    int64_t fit = avail > kCounterBytes ? (avail - kCounterBytes) / per_split : 1;
+    fit = std::max<int64_t>(1, std::min<int64_t>(fit, *splits));
+    const int64_t rpb = cdiv(cdiv(k, fit), granule) * granule;
+    *rows_per_block = int(rpb);
+    *splits = int(cdiv(k, rpb));
+}
+
 }  // namespace qmm

@@ -199,15 +199,11 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     int rpb, splits, tiles;
     skinny_plan(k, n, 512, parallel_k_parts, 128, &rpb, &splits, &tiles);
     QMM_CHECK(tiles <= kMaxSkinnyTiles, "N too large for the split-K counters");
+    skinny_fit_workspace(k, 128, tiles, int(std::min<int64_t>(16, m)), workspace, workspace_bytes, false, &rpb, &splits);
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16);
     const int grid = int(cdiv(tiles, 8) * 8 * splits);
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
-        if (splits > 1) {
-            const int64_t need = kCounterBytes + int64_t(tiles) * splits * mt * kSkinnyTileN * 4;
-            QMM_CHECK(workspace && workspace_bytes >= need,
-                      "workspace too small: need " << need << " bytes, got " << workspace_bytes);
-        }
         float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
         uint32_t *counters = static_cast<uint32_t *>(workspace);
         const size_t shmem = skinny_lds_bytes(mt);

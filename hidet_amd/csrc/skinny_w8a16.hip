@@ -129,7 +129,8 @@ __global__ __launch_bounds__(256) void naive_w8a16_kernel(const _Float16 *__rest
 }  // namespace
 
 void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace,
+                         hipStream_t stream) {
     const bool fast = (n % 16 == 0) && aligned(w, 16) && aligned(c, 8) && k > 0;  // 8-byte output stores in the split-K sum
     if (!fast) {
         launch(naive_w8a16_kernel, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, static_cast<const _Float16 *>(a), lda,
@@ -139,15 +140,11 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
     int rpb, splits, tiles;
     skinny_plan(k, n, m > 8 ? 768 : 512, parallel_k_parts, 128, &rpb, &splits, &tiles);
     QMM_CHECK(tiles <= kMaxSkinnyTiles, "N too large for the split-K counters");
+    skinny_fit_workspace(k, 128, tiles, int(std::min<int64_t>(16, m)), workspace, workspace_bytes, strict_workspace, &rpb, &splits);
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16);
     const int grid = int(cdiv(tiles, 8) * 8 * splits);
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
-        if (splits > 1) {
-            const int64_t need = kCounterBytes + int64_t(tiles) * splits * mt * kTileN * 4;
-            QMM_CHECK(workspace && workspace_bytes >= need,
-                      "workspace too small: need " << need << " bytes, got " << workspace_bytes);
-        }
         float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
         uint32_t *counters = static_cast<uint32_t *>(workspace);
         const _Float16 *ap = static_cast<const _Float16 *>(a) + m0 * lda;

@@ -51,7 +51,9 @@ const char *hidet_get_last_error(void);
 /* ---- library facts ---------------------------------------------------------------------------*/
 int hidet_qmm_abi_version(void);
 const char *hidet_qmm_arch(void);            /* "gfx950" */
-int64_t hidet_qmm_min_workspace_bytes(void); /* a workspace of this size serves every entry point */
+/* A workspace of this size lets every entry point use the K split it would choose for the shapes of a 4096- to 8192-wide
+ * transformer; with less (or with very wide outputs) the kernels use fewer K slices, down to none, never an error. */
+int64_t hidet_qmm_min_workspace_bytes(void);
 
 /* ---- timing hook (measurement only) ----------------------------------------------------------
  * hidet_qmm_arm_timing makes the NEXT compute-kernel launch issued from this thread record its

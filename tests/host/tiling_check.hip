@@ -75,8 +75,39 @@ static int check_skinny(long long k, long long ncols, int slice_rows, int hint, 
     return 0;
 }
 
+// A plan cut down to a workspace: still whole granules covering K once, never more bytes than the workspace holds, the
+// plan untouched when it fits, and a strict caller gets an error exactly when it does not.
+static int check_fit(long long k, long long ncols, int rows, long long workspace_bytes) {
+    int rpb = 0, splits = 0, tiles = 0;
+    skinny_plan(k, ncols, rows > 8 ? 768 : 512, 0, 128, &rpb, &splits, &tiles);
+    const int rpb0 = rpb, splits0 = splits;
+    char dummy = 0;
+    const bool fits = skinny_workspace_need(tiles, splits, rows) <= workspace_bytes;
+    bool threw = false;
+    try {
+        int r2 = rpb, s2 = splits;
+        skinny_fit_workspace(k, 128, tiles, rows, &dummy, workspace_bytes, true, &r2, &s2);
+    } catch (const Error &) { threw = true; }
+    if (threw == fits) return std::printf("fit k=%lld n=%lld rows=%d ws=%lld: strict error %d, fits %d\n", k, ncols, rows, workspace_bytes, threw, fits), 1;
+    skinny_fit_workspace(k, 128, tiles, rows, &dummy, workspace_bytes, false, &rpb, &splits);
+    if (fits && (rpb != rpb0 || splits != splits0)) return std::printf("fit k=%lld n=%lld: a plan that fits was changed\n", k, ncols), 1;
+    if (rpb <= 0 || rpb % 128 != 0 || splits < 1 || splits > splits0 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
+        skinny_workspace_need(tiles, splits, rows) > workspace_bytes)
+        return std::printf("fit k=%lld n=%lld rows=%d ws=%lld: rows %d x %d splits need %lld\n", k, ncols, rows, workspace_bytes, rpb, splits,
+                           (long long)skinny_workspace_need(tiles, splits, rows)), 1;
+    return 0;
+}
+
 int main() {
     long long n = 0;
+    // 16384 x 128256 with 8 rows (an lm_head decode batch) wants 131 MB of partial tiles: it must come out within 64 MiB
+    for (long long ws : {0LL, 1024LL, 65536LL, 65536LL + 8192, 1LL << 20, 16LL << 20, (16LL << 20) + 65536, 64LL << 20})
+        for (long long k : {128LL, 4096LL, 11008LL, 16384LL})
+            for (long long nc : {256LL, 4096LL, 11008LL, 128256LL})
+                for (int rows : {1, 8, 16}) {
+                    if (check_fit(k, nc, rows, ws)) return 1;
+                    ++n;
+                }
     for (long long k : {32LL, 96LL, 128LL, 1000LL, 4096LL, 11008LL, 8192LL, 28672LL})
         for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL})
             for (int hint : {0, 1, 3, 8, 64})

@@ -125,15 +125,20 @@ def test_strided_rows_and_unaligned_shapes():
         assert O.max_rel_err(got, clib.quant_matmul_f32acc(a, q, s)) <= 2e-3, (m, k, n)
 
 
-def test_workspace_too_small_is_reported():
-    announce('w8a16 small workspace')
-    a, q, s = _case(0, 1, 4096, 4096)
+@pytest.mark.parametrize('ws_bytes', [0, 1024, (64 << 10) + (512 << 10)])
+def test_small_workspace_means_fewer_k_slices(ws_bytes):
+    # the plan for 8 x 4096 x 4096 wants 8 K slices = 64 KiB of counters + 1 MiB of partial tiles; with less the
+    # launcher takes the K split that fits (none without a workspace) and the result stays exact
+    announce('w8a16 small workspace', ws_bytes)
+    m, k, n = 8, 4096, 4096
+    a, q, s = _int_case(77, m, k, n)
+    want = ((a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :])
     ta, tq, ts = dev(a), dev(q), dev(s)
-    c = torch.empty(1, 4096, dtype=torch.float16, device='cuda')
-    ws = torch.zeros(1024, dtype=torch.uint8, device='cuda')
-    with pytest.raises(hidet_amd.BackendException, match='workspace too small'):
-        hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8', ta, tq, ts, c, 1, 4096, 4096, 4096, 0, ws, ws.numel(),
-                           hidet_amd.ffi.current_stream(ta.device))
+    c = torch.full((m, n), float('nan'), dtype=torch.float16, device='cuda')
+    ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device='cuda')
+    hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8', ta, tq, ts, c, m, k, n, k, 0, ws if ws_bytes else None,
+                       ws_bytes, hidet_amd.ffi.current_stream(ta.device))
+    assert np.array_equal(host(c), want.astype(np.float32).astype(np.float16))
 
 
 # ---- prefill GEMM (M > 16 goes to the MFMA kernel) ------------------------------------------------------------
