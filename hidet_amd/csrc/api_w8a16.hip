@@ -45,6 +45,33 @@ void w8a16_dispatch(const void *a, const void *w, const void *scale, void *c, in
                             stream);
 }
 
+// Scratch memory of hidet_symmetric_quant_matmul_f16_i8_static: arrival counters in the first 64 KiB, partial tiles
+// behind them; the layout a caller's workspace has. One copy per GPU, loaded with the library's code object (zero-filled
+// then; the kernels return every counter they used to zero).
+constexpr int64_t kStaticScratchBytes = HIDET_QMM_STATIC_SCRATCH_BYTES;
+static_assert(kStaticScratchBytes > kCounterBytes && kStaticScratchBytes % 256 == 0, "counters plus partial tiles");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, looked up on the first call there
+std::mutex g_scratch_mu;
+
+// The device address of this GPU's copy of `scratch`. In host code the array's name is only a handle for the runtime's
+// symbol lookup, never a pointer a kernel may be given.
+void *static_scratch_of_current_device() {
+    int device = -1;
+    QMM_HIP(hipGetDevice(&device));
+    QMM_CHECK(device >= 0 && device < kMaxDevices, "device ordinal " << device << " out of range");
+    std::lock_guard<std::mutex> guard(g_scratch_mu);
+    if (g_scratch_ptr[device] == nullptr) {
+        void *ptr = nullptr;
+        QMM_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        QMM_CHECK(ptr != nullptr && aligned(ptr, 256), "the runtime returned no usable address for the static scratch array");
+        g_scratch_ptr[device] = ptr;
+    }
+    return g_scratch_ptr[device];
+}
+
 }  // namespace
 
 HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
@@ -52,6 +79,18 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
                                                    void *workspace, int64_t workspace_bytes, void *stream_) {
     QMM_ENTRY_BEGIN
     w8a16_dispatch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, false,
+                   static_cast<hipStream_t>(stream_));
+    QMM_ENTRY_END
+}
+
+HIDET_API int64_t hidet_qmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+HIDET_API void hidet_symmetric_quant_matmul_f16_i8_static(const void *a, const void *w, const void *scale, void *c, int64_t m,
+                                                          int64_t k, int64_t n, int64_t lda, int parallel_k_parts,
+                                                          void *stream_) {
+    QMM_ENTRY_BEGIN
+    void *ptr = static_scratch_of_current_device();
+    w8a16_dispatch(a, w, scale, c, m, k, n, lda, parallel_k_parts, ptr, kStaticScratchBytes, true,
                    static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

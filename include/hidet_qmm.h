@@ -93,6 +93,20 @@ void hidet_symmetric_dequantize(const void *wq, const void *scale, void *w, int6
 void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
                                          int64_t k, int64_t n, int64_t lda, int parallel_k_parts, void *workspace,
                                          int64_t workspace_bytes, void *stream);
+/* The same operator for callers that can neither allocate device memory nor pass a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose tasks
+ * take their scratch from the runtime's grow-only request_hip_workspace).  Same arguments, checks, kernels and results
+ * as hidet_symmetric_quant_matmul_f16_i8 called with a workspace of HIDET_QMM_STATIC_SCRATCH_BYTES; the scratch memory
+ * is an array of that size inside the library's device code, one copy per GPU for the life of the process.  The call
+ * allocates and frees nothing.  Up to 16 rows (and whenever the bandwidth-bound kernel is chosen) a shape whose K split
+ * needs more partial-tile memory than the array holds is rejected with an error that names the bytes needed; taller
+ * matrices always run, in as many K ranges as fit.  Every call on one GPU uses the same array: calls that overlap in
+ * time on one GPU (two streams, two threads) race; calls ordered by a stream or by events do not.  The device the
+ * stream belongs to must be current. */
+#define HIDET_QMM_STATIC_SCRATCH_BYTES ((16 << 20) + (64 << 10))
+int64_t hidet_qmm_static_scratch_bytes(void);
+void hidet_symmetric_quant_matmul_f16_i8_static(const void *a, const void *w, const void *scale, void *c, int64_t m,
+                                                int64_t k, int64_t n, int64_t lda, int parallel_k_parts, void *stream);
 /* The same operator for a weight that is stored K-contiguous: w_nk[n * ldw + k] = w[k, n] (the [K, N] operand held
  * with strides (1, ldw); what torch's nn.Linear keeps, and what a matmul with transpose_b=True reads,
  * python/hidet/graph/ops/matmul/matmul.py:37-38, python/hidet/graph/frontend/torch/register_functions.py:165-167).
