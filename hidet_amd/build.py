@@ -20,6 +20,9 @@ FLAGS = [
     '--offload-arch=' + ARCH, '-O3', '-std=c++17', '-fPIC', '-fvisibility=hidden',
     # keep the compiler from forming packed-fp32 instructions
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+    # kernel arguments arrive in scalar registers with the wave instead of being fetched by its first instructions
+    # (a kernel's first load waits about 0.3 us less; the code falls back to fetching them where that is not supported)
+    '-mllvm', '-amdgpu-kernarg-preload-count=16',
 ]
 
 

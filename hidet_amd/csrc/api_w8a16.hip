@@ -45,9 +45,9 @@ void w8a16_dispatch(const void *a, const void *w, const void *scale, void *c, in
                             stream);
 }
 
-// Scratch memory of hidet_symmetric_quant_matmul_f16_i8_static: arrival counters in the first 64 KiB, partial tiles
-// behind them; the layout a caller's workspace has. One copy per GPU, loaded with the library's code object (zero-filled
-// then; the kernels return every counter they used to zero).
+// Scratch memory of hidet_symmetric_quant_matmul_f16_i8_static, used exactly like a caller's workspace of that size
+// (counters, mailbox, scratch). One copy per GPU, loaded with the library's code object (zero-filled then; the kernels
+// return every counter and every mailbox word they used to zero).
 constexpr int64_t kStaticScratchBytes = HIDET_QMM_STATIC_SCRATCH_BYTES;
 static_assert(kStaticScratchBytes > kCounterBytes && kStaticScratchBytes % 256 == 0, "counters plus partial tiles");
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];

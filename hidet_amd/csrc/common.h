@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <exception>
 #include <mutex>
@@ -128,9 +129,33 @@ typedef int int8v_t __attribute__((ext_vector_type(8)));
 typedef int int4v_t __attribute__((ext_vector_type(4)));
 typedef unsigned int uint4v_t __attribute__((ext_vector_type(4)));
 
-// The first 64 KiB of a caller-provided workspace hold arrival counters of cross-workgroup exchanges (always
-// returned to zero by the kernel that used them); scratch for partial results follows.
+// A caller-provided workspace has three parts. The first 64 KiB hold arrival counters of cross-workgroup exchanges
+// (always returned to zero by the kernel that used them). The mailbox behind them - a quarter of the rest, at most
+// 16 MiB - belongs to the split-K exchange of the bandwidth-bound kernels, which finds it all zero and leaves it all
+// zero. What follows is plain scratch (partial tiles of the GEMMs, column maxima of the quantizers) whose contents
+// nobody relies on between launches.
 constexpr int64_t kCounterBytes = 64 << 10;
+constexpr int64_t kMaxMailboxBytes = 16 << 20;
+
+struct Workspace {
+    uint32_t *counters = nullptr;
+    float *mailbox = nullptr;
+    int64_t mailbox_bytes = 0;
+    char *scratch = nullptr;
+    int64_t scratch_bytes = 0;
+};
+
+inline Workspace split_workspace(void *workspace, int64_t bytes) {
+    Workspace v;
+    if (workspace == nullptr || bytes < kCounterBytes) return v;
+    const int64_t rest = bytes - kCounterBytes;
+    v.counters = static_cast<uint32_t *>(workspace);
+    v.mailbox_bytes = std::min(kMaxMailboxBytes, rest / 4) / 256 * 256;
+    v.mailbox = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
+    v.scratch = static_cast<char *>(workspace) + kCounterBytes + v.mailbox_bytes;
+    v.scratch_bytes = rest - v.mailbox_bytes;
+    return v;
+}
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(static_cast<uint32_t>(b) << 16); }
 

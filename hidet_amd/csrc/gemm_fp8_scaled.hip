@@ -439,11 +439,12 @@ static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ld
     const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
     // Tail split (tiles that do not fill a round of one workgroup per CU are computed in K ranges and summed in range
     // order by the last workgroup to arrive): at most 4 ranges of at least 4 k blocks, and only with a workspace that
-    // holds the partial tiles (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
+    // holds the partial tiles (8 XCDs x their tail tiles x parts) in its scratch part.
     GemmTail tail = make_gemm_tail(tiling, 32, 32, 4);
-    if (workspace == nullptr || workspace_bytes < kCounterBytes) tail.parts = 1;
-    while (tail.parts > 1 && (k / 128 < 4 * tail.parts ||
-                              workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * kM8 * kN8 * 4))
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
+    if (ws.scratch == nullptr) tail.parts = 1;
+    while (tail.parts > 1 &&
+           (k / 128 < 4 * tail.parts || ws.scratch_bytes < int64_t(8) * tail.max_tiles * tail.parts * kM8 * kN8 * 4))
         --tail.parts;
     const int64_t grid = gemm_grid_with_tail(tiling, 32, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
@@ -452,7 +453,7 @@ static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ld
         launch(kern, dim3(uint32_t(grid)), dim3(kThreads8), size_t(kLdsBytes8), stream, static_cast<const uint8_t *>(a), lda,
                static_cast<const uint8_t *>(b), ldb, static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
                int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn, tail.parts, tail.max_tiles,
-               reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
+               reinterpret_cast<float *>(ws.scratch), ws.counters);
     };
     switch (out_dtype) {
         case HIDET_QMM_F32: go(gemm_fp8_kernel8<HIDET_QMM_F32, SCALED>); break;

@@ -453,9 +453,9 @@ void launch_cfg16(const void *a, const void *w, const void *scales, void *c, int
     constexpr int kConcurrent = 32 * MIN_BLOCKS;
     const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
     GemmTail tail = make_gemm_tail(tiling, kConcurrent, kConcurrent, 4);
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
     while (tail.parts > 1 &&
-           (k / kBK < 8 * tail.parts ||
-            workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
+           (k / kBK < 8 * tail.parts || ws.scratch_bytes < int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
         --tail.parts;
     const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
@@ -463,8 +463,7 @@ void launch_cfg16(const void *a, const void *w, const void *scales, void *c, int
     launch(gemm_w4a16_kernel16<DT, RB, WM, WN, MIN_BLOCKS>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes),
            stream, static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
            static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,
-           tail.parts, tail.max_tiles, reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes),
-           static_cast<uint32_t *>(workspace));
+           tail.parts, tail.max_tiles, reinterpret_cast<float *>(ws.scratch), ws.counters);
 }
 
 
@@ -821,9 +820,9 @@ void launch_lds(const void *a, const void *w, const void *scales, void *c, int64
     // time is about 74 us at K = 4096 (measured: M = 512, all 172 tiles in 4 parts: 82 -> 104 us; M = 1024, 88 tail
     // tiles in 2 parts: 146 -> 121 us)
     GemmTail tail = make_gemm_tail_by_rounds(tiling, kConcurrent, 4, 0.0007 * 4096.0 / double(k));
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
     while (tail.parts > 1 &&
-           (k / kBK < 8 * tail.parts ||
-            workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
+           (k / kBK < 8 * tail.parts || ws.scratch_bytes < int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
         --tail.parts;
     const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
@@ -831,8 +830,7 @@ void launch_lds(const void *a, const void *w, const void *scales, void *c, int64
     launch(gemm_w4a16_lds_kernel<DT>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
            static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,
-           tail.parts, tail.max_tiles, reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes),
-           static_cast<uint32_t *>(workspace));
+           tail.parts, tail.max_tiles, reinterpret_cast<float *>(ws.scratch), ws.counters);
 }
 
 }  // namespace

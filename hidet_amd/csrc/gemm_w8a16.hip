@@ -308,7 +308,7 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     constexpr int kConcurrent = 32 * MIN_BLOCKS;  // workgroups an XCD (32 CUs) runs at a time
     const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, kConcurrent);
     // Tail split: at most 4 K ranges of at least 8 stages each, and only with workspace for the partial tiles
-    // (8 XCDs x their tail tiles x parts) behind the 64 KiB of counters.
+    // (8 XCDs x their tail tiles x parts) in the scratch part of the workspace.
     // (light workgroups - at most 4 active row blocks - are worth up to 8 ranges: measured)
     GemmTail tail = make_gemm_tail(tiling, kConcurrent, 32, RBA <= 4 ? 8 : 4);
     // Full tiles: count rounds of one workgroup per CU. The tiles past a whole number of such rounds share their CUs
@@ -320,9 +320,9 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
         tail = make_gemm_tail_by_rounds(tiling, 32, 4, 0.00085 * 4096.0 / double(k));
         split_unit = 32;
     }
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
     while (tail.parts > 1 &&
-           (k / kBK < 8 * tail.parts ||
-            workspace_bytes < kCounterBytes + int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
+           (k / kBK < 8 * tail.parts || ws.scratch_bytes < int64_t(8) * tail.max_tiles * tail.parts * Cfg::kBM * Cfg::kBN * 4))
         --tail.parts;
     static_assert(8 * kConcurrent * 4 <= kCounterBytes, "one counter per tail tile");
     const int64_t grid = gemm_grid_with_tail(tiling, split_unit, tail);
@@ -331,7 +331,7 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA, W_NK>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale),
            static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, split_unit, tail.parts, tail.max_tiles,
-           reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes), static_cast<uint32_t *>(workspace));
+           reinterpret_cast<float *>(ws.scratch), ws.counters);
 }
 
 }  // namespace

@@ -527,10 +527,11 @@ HIDET_API void hidet_symmetric_quantize(const void *w, void *wq, void *scale, in
     if (nscale == 0) return;
     QMM_CHECK(scale && (total == 0 || (w && wq)), "null tensor pointer");
     QMM_CHECK(inner < (int64_t(1) << 31) * 64 && outer < 65536 * int64_t(4), "extent too large");
-    QMM_CHECK(workspace && workspace_bytes >= kCounterBytes + nscale * 4,
-              "workspace too small: need " << kCounterBytes + nscale * 4 << " bytes, got " << workspace_bytes);
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
+    QMM_CHECK(ws.scratch_bytes >= nscale * 4, "workspace too small: its scratch part (three quarters of what follows the first 64 KiB) must hold "
+                                                  << nscale * 4 << " bytes, got a workspace of " << workspace_bytes);
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    uint32_t *amax_bits = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kCounterBytes);
+    uint32_t *amax_bits = reinterpret_cast<uint32_t *>(ws.scratch);
     dispatch_float(w_dtype, [&](auto dt) {
         constexpr int DT = decltype(dt)::value;
         {
@@ -665,10 +666,11 @@ HIDET_API void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *s
                                              void *workspace, int64_t workspace_bytes, void *stream_) {
     QMM_ENTRY_BEGIN
     QMM_CHECK(scale, "null scale pointer");
-    QMM_CHECK(workspace && workspace_bytes >= kCounterBytes + 4, "workspace too small");
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
+    QMM_CHECK(ws.scratch_bytes >= 4, "workspace too small");
     QMM_CHECK(numel == 0 || (x && codes), "null tensor pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    uint32_t *amax_bits = reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + kCounterBytes);
+    uint32_t *amax_bits = reinterpret_cast<uint32_t *>(ws.scratch);
     dispatch_float(x_dtype, [&](auto dt) {
         constexpr int DT = decltype(dt)::value;
         const int esize = DT == HIDET_QMM_F32 ? 4 : 2;

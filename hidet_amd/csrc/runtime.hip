@@ -36,7 +36,7 @@ HIDET_API const char *hidet_get_last_error(void) {
 
 HIDET_API int hidet_qmm_abi_version(void) { return HIDET_QMM_ABI_VERSION; }
 HIDET_API const char *hidet_qmm_arch(void) { return "gfx950"; }
-HIDET_API int64_t hidet_qmm_min_workspace_bytes(void) { return int64_t(64) << 20; }
+HIDET_API int64_t hidet_qmm_min_workspace_bytes(void) { return int64_t(96) << 20; }
 
 HIDET_API void *hidet_qmm_event_create(void) {
     hipEvent_t e = nullptr;

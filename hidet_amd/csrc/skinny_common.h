@@ -1,17 +1,15 @@
-// Shared tail of the bandwidth-bound skinny kernels (M <= 16 rows per pass, 256-column tiles, 4 waves
-// per workgroup that split K): LDS reduction over the waves, then either a direct store or the
-// cross-workgroup split-K exchange.
+// Shared parts of the bandwidth-bound skinny kernels (M <= 16 rows per pass, 256-column tiles, the waves of a
+// workgroup split its K slice): the launch plan, the LDS reduction over the waves and the split-K exchange
+// between workgroups.
 #pragma once
 #include "common.h"
 
 namespace qmm {
 
 constexpr int kSkinnyTileN = 256;
-constexpr int kSkinnyWaves = 4;
 constexpr int kSkinnyRedStride = 272;  // 16 lanes x 17 floats: conflict-free LDS writes
-constexpr int kMaxSkinnyTiles = int(kCounterBytes / 4);
 
-inline size_t skinny_lds_bytes(int m) { return size_t(kSkinnyWaves) * m * kSkinnyRedStride * sizeof(float); }
+inline size_t skinny_lds_bytes(int m, int waves) { return size_t(waves) * m * kSkinnyRedStride * sizeof(float); }
 
 template <typename OutT>
 __device__ __forceinline__ OutT skinny_to_out(float v);
@@ -34,20 +32,228 @@ __device__ __forceinline__ bool skinny_tile_of_block(int splits, int tiles, int 
     return skinny_tile_of(int(blockIdx.x), splits, tiles, tile, split);
 }
 
-// res[t][v] is this lane's partial sum for output row 4 * (lane / 16) + v and column
-// tile * 256 + (lane % 16) * 16 + t.  `red` is dynamic LDS of skinny_lds_bytes(m).
-// col_scale (may be null) is a per-column float16 factor applied to the final sum.
+// The tail of a bandwidth-bound kernel: LDS reduction over the WAVES waves of a workgroup, then either the final store or
+// the split-K exchange through the mailbox.
 //
-// Cross-workgroup exchange without cache-wide fences: a partial tile is written with agent-scope
-// (write-through) stores, their completion is awaited, and only then is the arrival counted; the
-// last workgroup to arrive reads all partial tiles back with agent-scope loads and adds them in
-// split order, so the result does not depend on arrival order.  A release/acquire fence pair here
-// would write back and invalidate the whole L2 once per workgroup, which costs more than the GEMV.
-template <typename OutT>
-__device__ __forceinline__ void skinny_reduce_store(const float4_t (&res)[16], int m, int n, int tile, int split,
-                                                    int splits, const _Float16 *__restrict__ col_scale,
-                                                    OutT *__restrict__ c, float *__restrict__ partials,
-                                                    uint32_t *__restrict__ counters, float *red, int *s_last) {
+// res[t][v] is this lane's partial sum for output row 4 * (lane / 16) + v and column tile * 256 + (lane % 16) * 16 + t.
+// `red` is dynamic LDS of skinny_lds_bytes(m, WAVES). col_scale points at the factors of the tile's 256 columns (or is
+// null); the factors a thread needs are fetched before the caller's main loop would be ideal, but they come from the
+// cache by the time the tail runs: the caller touches them early (skinny_prefetch_scale).
+//
+// Who does what in the tail: with up to 4 rows thread tid owns column tid % 256 of rows tid / 256, tid / 256 + WAVES / 4,
+// ... (one dword per access, four waves per row); with more rows it owns columns 4 (tid % 64) .. + 3 of rows tid / 64,
+// tid / 64 + WAVES, ... (16 bytes per access, one wave per row). Either way every wave has work: the same bytes moved
+// by a single wave were measured 1 us slower per launch, and every batch of reads from the mailbox costs a round trip
+// to the memory side (1.5 to 2 us), so a thread wants all its reads in one batch of 16.
+//
+// Exchange: the mailbox holds one fp32 tile [m][256] per (column tile, K slice) and is all zero between launches. Every
+// slice but the last stores its tile (agent scope, +0.0 sent as -0.0, so a stored word is never zero) and is done: no
+// acknowledgement, no counter. The workgroup of the LAST slice - the highest workgroup index of the column tile, so all
+// the others were dispatched before it - reads the tiles back until no word is zero, adds them in slice order (its own
+// last: the result does not depend on timing), writes the output and puts the zeros back with plain stores, which the
+// end of the kernel makes visible to the next launch. The wait is bounded: after kSkinnySpinLimit re-reads the output
+// is NaN instead of a hang.
+constexpr int kSkinnySpinLimit = 1 << 20;
+
+// Column factors of a thread for both thread layouts of the tail, fetched by the caller before its main loop and not
+// looked at there (a use would make the first weight load wait for them).
+struct SkinnyScale {
+    _Float16 one = _Float16(1.0f);                                                    // column tid % 256
+    half4_t quad = {_Float16(1.0f), _Float16(1.0f), _Float16(1.0f), _Float16(1.0f)};  // columns 4 (tid % 64) .. + 3
+};
+__device__ __forceinline__ SkinnyScale skinny_fetch_scale(const _Float16 *scale, int tile_col, int n, int m) {
+    SkinnyScale s;
+    const int tid = threadIdx.x;
+    if (m <= 4) {
+        if (tile_col + (tid & 255) < n) s.one = scale[tile_col + (tid & 255)];
+    } else {
+        if (tile_col + (tid & 63) * 4 < n) s.quad = *reinterpret_cast<const half4_t *>(scale + tile_col + (tid & 63) * 4);
+    }
+    return s;
+}
+
+// CW columns per thread: the word a thread moves is one dword or four. Agent scope (sc1): loads bypass the L1, stores
+// write through.
+template <int CW>
+struct SkinnyWord;
+template <>
+struct SkinnyWord<1> {
+    typedef uint32_t type;
+    static __device__ __forceinline__ type absent() { return 0x80000000u; }  // -0.0: adds nothing, counts as arrived
+    static __device__ __forceinline__ bool has_zero(type v) { return v == 0u; }
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 1 << 4); }
+    static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, int off, type v) { __builtin_amdgcn_raw_buffer_store_b32(v, r, off, 0, 1 << 4); }
+    static __device__ __forceinline__ void clear(__amdgpu_buffer_rsrc_t r, int off) { __builtin_amdgcn_raw_buffer_store_b32(0u, r, off, 0, 0); }
+    static __device__ __forceinline__ type never_zero(type v) { return v == 0u ? 0x80000000u : v; }
+    static __device__ __forceinline__ float get(type v, int) { return __uint_as_float(v); }
+};
+template <>
+struct SkinnyWord<4> {
+    typedef uint4v_t type;
+    static __device__ __forceinline__ type absent() { return type{0x80000000u, 0x80000000u, 0x80000000u, 0x80000000u}; }
+    static __device__ __forceinline__ bool has_zero(type v) { return v[0] == 0u || v[1] == 0u || v[2] == 0u || v[3] == 0u; }
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int off) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 1 << 4); }
+    static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, int off, type v) { __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, 1 << 4); }
+    static __device__ __forceinline__ void clear(__amdgpu_buffer_rsrc_t r, int off) { __builtin_amdgcn_raw_buffer_store_b128(type{0u, 0u, 0u, 0u}, r, off, 0, 0); }
+    static __device__ __forceinline__ type never_zero(type v) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (v[e] == 0u) v[e] = 0x80000000u;
+        return v;
+    }
+    static __device__ __forceinline__ float get(type v, int e) { return __uint_as_float(v[e]); }
+};
+
+template <typename OutT, int WAVES, int CW>
+struct SkinnyTail {
+    typedef SkinnyWord<CW> W;
+    typedef typename W::type Word;
+    static constexpr int kThreadsPerRow = kSkinnyTileN / CW;                // 256 or 64
+    static constexpr int kRowGroups = WAVES * 64 / kThreadsPerRow;         // rows the workgroup handles at a time
+    static_assert(WAVES % 4 == 0, "whole rows of threads");
+    int m, n, row_first, col_in_tile;
+    int64_t out_col;
+    const float *red;
+    float scale[CW];
+    OutT *c;
+
+    struct Vals {
+        float v[CW];
+    };
+    __device__ __forceinline__ Vals own(int row) const {
+        const float *src = red + row * kSkinnyRedStride + col_in_tile + (col_in_tile >> 4);  // CW columns never straddle 16
+        Vals r;
+#pragma unroll
+        for (int e = 0; e < CW; ++e) r.v[e] = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv)
+#pragma unroll
+            for (int e = 0; e < CW; ++e) r.v[e] += src[wv * m * kSkinnyRedStride + e];
+        return r;
+    }
+    __device__ __forceinline__ void store(int row, const Vals &x) const {
+        OutT *dst = c + int64_t(row) * n + out_col;
+        if constexpr (CW == 1) {
+            dst[0] = skinny_to_out<OutT>(x.v[0] * scale[0]);
+        } else {
+            uint16_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, skinny_to_out<OutT>(x.v[e] * scale[e]));
+            // 8 bytes at once when the row starts allow it (n a multiple of 4 is given, the base pointer may not be aligned)
+            if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+                *reinterpret_cast<uint2 *>(dst) = uint2{uint32_t(h[0]) | (uint32_t(h[1]) << 16), uint32_t(h[2]) | (uint32_t(h[3]) << 16)};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) reinterpret_cast<uint16_t *>(dst)[e] = h[e];
+            }
+        }
+    }
+    static __device__ __forceinline__ Word pack(const Vals &x) {
+        if constexpr (CW == 1) {
+            return W::never_zero(__float_as_uint(x.v[0]));
+        } else {
+            return W::never_zero(Word{__float_as_uint(x.v[0]), __float_as_uint(x.v[1]), __float_as_uint(x.v[2]), __float_as_uint(x.v[3])});
+        }
+    }
+
+    // A slice that is not the last: send the partial tile.
+    __device__ __forceinline__ void send(__amdgpu_buffer_rsrc_t box, int split) const {
+#pragma unroll 1
+        for (int row = row_first; row < m; row += kRowGroups)
+            W::store(box, ((split * m + row) * kSkinnyTileN + col_in_tile) * 4, pack(own(row)));
+    }
+
+    // The last slice: 16 reads in flight, (16 >> LG) rows x (1 << LG) slices per trip.
+    template <int LG>
+    __device__ __forceinline__ void collect(__amdgpu_buffer_rsrc_t box, int others) const {
+        constexpr int kRows = 16 >> LG, kSlices = 1 << LG;
+#pragma unroll 1
+        for (int row0 = row_first; row0 < m; row0 += kRows * kRowGroups) {
+            Vals total[kRows];
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                if (row0 + r * kRowGroups < m) total[r] = own(row0 + r * kRowGroups);
+                else
+#pragma unroll
+                    for (int e = 0; e < CW; ++e) total[r].v[e] = 0.f;
+            }
+            bool lost = false;
+            // the sum runs over the slices in order and ends with this workgroup's own part: keep `total` for last
+            Vals others_sum[kRows];
+#pragma unroll
+            for (int r = 0; r < kRows; ++r)
+#pragma unroll
+                for (int e = 0; e < CW; ++e) others_sum[r].v[e] = 0.f;
+#pragma unroll 1
+            for (int sp0 = 0; sp0 < others; sp0 += kSlices) {
+                Word bits[16];
+                int off[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    const int row = row0 + (u >> LG) * kRowGroups, sp = sp0 + (u & (kSlices - 1));
+                    off[u] = (row < m && sp < others) ? ((sp * m + row) * kSkinnyTileN + col_in_tile) * 4 : -1;
+                    bits[u] = W::absent();
+                    if (off[u] >= 0) bits[u] = W::load(box, off[u]);
+                }
+#pragma unroll 1
+                for (int spin = 0;; ++spin) {
+                    bool missing = false;
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) missing |= W::has_zero(bits[u]);
+                    if (!missing) break;
+                    if (spin == kSkinnySpinLimit) {
+                        lost = true;
+                        break;
+                    }
+                    asm volatile("" ::: "memory");  // the mailbox changes under the loop: the reads below are issued again
+#pragma unroll
+                    for (int u = 0; u < 16; ++u)
+                        if (W::has_zero(bits[u])) bits[u] = W::load(box, off[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+#pragma unroll
+                    for (int e = 0; e < CW; ++e) others_sum[u >> LG].v[e] += W::get(bits[u], e);
+                    if (off[u] >= 0) W::clear(box, off[u]);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                const int row = row0 + r * kRowGroups;
+                if (row < m) {
+                    Vals out;
+#pragma unroll
+                    for (int e = 0; e < CW; ++e) out.v[e] = lost ? __builtin_nanf("") : others_sum[r].v[e] + total[r].v[e];
+                    store(row, out);
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void run(int tile, int split, int splits, float *mailbox) const {
+        if (splits == 1) {
+#pragma unroll 1
+            for (int row = row_first; row < m; row += kRowGroups) store(row, own(row));
+            return;
+        }
+        const int others = splits - 1;
+        const __amdgpu_buffer_rsrc_t box = __builtin_amdgcn_make_buffer_rsrc(mailbox + int64_t(tile) * splits * m * kSkinnyTileN, 0,
+                                                                             others * m * kSkinnyTileN * 4, 0x00020000);
+        if (split != others) {
+            send(box, split);
+            return;
+        }
+        const int my_rows = (m - row_first + kRowGroups - 1) / kRowGroups;
+        if (others <= 4 && my_rows > 2) collect<2>(box, others);
+        else if (others <= 8 && my_rows > 1) collect<3>(box, others);
+        else collect<4>(box, others);
+    }
+};
+
+template <typename OutT, int WAVES>
+__device__ __forceinline__ void skinny_finish(const float4_t (&res)[16], int m, int n, int tile, int split, int splits,
+                                              const SkinnyScale &col_scale, OutT *__restrict__ c, float *__restrict__ mailbox,
+                                              float *red) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 4, cl = lane & 15;
@@ -62,102 +268,30 @@ __device__ __forceinline__ void skinny_reduce_store(const float4_t (&res)[16], i
     }
     __syncthreads();
 
-    const int col = tile * kSkinnyTileN + tid;
-    const int ridx = tid + (tid >> 4);
-    const float s = (col_scale != nullptr && col < n) ? float(col_scale[col]) : 1.0f;
-    if (splits == 1) {
-        if (col < n) {
-            for (int row = 0; row < m; ++row) {
-                float v = 0.f;
+    if (m <= 4) {
+        SkinnyTail<OutT, WAVES, 1> tail;
+        tail.m = m;
+        tail.n = n;
+        tail.row_first = __builtin_amdgcn_readfirstlane(tid >> 8);  // the same for a whole wave: row and slice tests are scalar
+        tail.col_in_tile = tid & 255;
+        tail.out_col = int64_t(tile) * kSkinnyTileN + tail.col_in_tile;
+        tail.red = red;
+        tail.scale[0] = float(col_scale.one);
+        tail.c = c;
+        if (tail.out_col < n && tail.row_first < m) tail.run(tile, split, splits, mailbox);
+    } else {
+        SkinnyTail<OutT, WAVES, 4> tail;
+        tail.m = m;
+        tail.n = n;
+        tail.row_first = __builtin_amdgcn_readfirstlane(tid >> 6);
+        tail.col_in_tile = (tid & 63) * 4;
+        tail.out_col = int64_t(tile) * kSkinnyTileN + tail.col_in_tile;
+        tail.red = red;
 #pragma unroll
-                for (int wv = 0; wv < kSkinnyWaves; ++wv) v += red[(wv * m + row) * kSkinnyRedStride + ridx];
-                c[int64_t(row) * n + col] = skinny_to_out<OutT>(v * s);
-            }
-        }
-        return;
+        for (int e = 0; e < 4; ++e) tail.scale[e] = float(col_scale.quad[e]);
+        tail.c = c;
+        if (tail.out_col < n && tail.row_first < m) tail.run(tile, split, splits, mailbox);  // n is a multiple of 16: a quad is in or out as a whole
     }
-
-    float *mine = partials + (int64_t(tile) * splits + split) * m * kSkinnyTileN;
-    for (int row = 0; row < m; ++row) {
-        float v = 0.f;
-#pragma unroll
-        for (int wv = 0; wv < kSkinnyWaves; ++wv) v += red[(wv * m + row) * kSkinnyRedStride + ridx];
-        __hip_atomic_store(mine + row * kSkinnyTileN + tid, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): every store of this lane has been acknowledged
-    __syncthreads();
-    if (tid == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *s_last = (old == uint32_t(splits - 1));
-    }
-    __syncthreads();
-    if (!*s_last) return;
-    if (col < n) {
-        const float *base = partials + int64_t(tile) * splits * m * kSkinnyTileN;
-        if (m == 1) {
-            float v = 0.f;
-            for (int sp0 = 0; sp0 < splits; sp0 += 16) {  // 16 loads in flight, added in split order
-                float part[16];
-#pragma unroll
-                for (int u = 0; u < 16; ++u) {
-                    part[u] = 0.f;
-                    if (sp0 + u < splits)
-                        part[u] = __hip_atomic_load(base + int64_t(sp0 + u) * kSkinnyTileN + tid, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-                }
-#pragma unroll
-                for (int u = 0; u < 16; ++u) v += part[u];
-            }
-            c[col] = skinny_to_out<OutT>(v * s);
-        }
-    }
-    if (m > 1) {
-        // 256 threads = 4 row lanes x 64 column quads: thread (rl, cq) sums rows rl, rl + 4, ... of columns 4cq .. 4cq+3
-        // with 16-byte agent-scope loads, two rows x eight splits = 16 loads in flight, each row added in split order.
-        const int cq = tid & 63, rl = tid >> 6;
-        const int col4 = tile * kSkinnyTileN + cq * 4;
-        if (col4 < n) {  // n is a multiple of 16 on this path: the quad is in or out as a whole
-            constexpr int kAgentScope = 1 << 4;  // sc1
-            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                partials + int64_t(tile) * splits * m * kSkinnyTileN, 0, splits * m * kSkinnyTileN * 4, 0x00020000);
-            float s4[4] = {1.f, 1.f, 1.f, 1.f};
-            if (col_scale != nullptr) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) s4[e] = float(col_scale[col4 + e]);
-            }
-            for (int row0 = rl; row0 < m; row0 += 8) {
-                float4_t v[2] = {float4_t{0.f, 0.f, 0.f, 0.f}, float4_t{0.f, 0.f, 0.f, 0.f}};
-                for (int sp0 = 0; sp0 < splits; sp0 += 8) {
-                    uint4v_t part[2][8];
-#pragma unroll
-                    for (int r = 0; r < 2; ++r)
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) {
-                            const int row = row0 + 4 * r, sp = sp0 + u;
-                            // past the last row or split: an offset outside the buffer, which reads as zero
-                            const int off = (row < m && sp < splits) ? ((sp * m + row) * kSkinnyTileN + cq * 4) * 4 : 0x7FFFFFF0;
-                            part[r][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kAgentScope);
-                        }
-#pragma unroll
-                    for (int r = 0; r < 2; ++r)
-#pragma unroll
-                        for (int u = 0; u < 8; ++u) v[r] += __builtin_bit_cast(float4_t, part[r][u]);
-                }
-#pragma unroll
-                for (int r = 0; r < 2; ++r) {
-                    const int row = row0 + 4 * r;
-                    if (row < m) {
-                        uint16_t h[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, skinny_to_out<OutT>(v[r][e] * s4[e]));
-                        *reinterpret_cast<uint2 *>(c + int64_t(row) * n + col4) =
-                            uint2{uint32_t(h[0]) | (uint32_t(h[1]) << 16), uint32_t(h[2]) | (uint32_t(h[3]) << 16)};
-                    }
-                }
-            }
-        }
-    }
-    if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next call
 }
 
 // K split of a skinny launch. Each workgroup streams a slice of `rows_per_block` weight rows (a whole multiple of
@@ -178,23 +312,37 @@ inline void skinny_plan(int64_t k, int64_t n, int slice_rows, int hint_parts, in
     *tiles = int(t);
 }
 
-// Bytes of workspace a skinny launch with `splits` K slices touches: the counters and one fp32 partial tile per
-// (column tile, K slice) of `rows` (at most 16) activation rows. One slice exchanges nothing.
-inline int64_t skinny_workspace_need(int tiles, int splits, int rows) {
-    return splits > 1 ? kCounterBytes + int64_t(tiles) * splits * rows * kSkinnyTileN * 4 : 0;
+// K split of the int8 kernel, whose workgroups have `waves` waves: one round of one workgroup per CU. Measured on
+// K = 4096 .. 14336, N = 1024 .. 32000: the fastest split is the largest whose workgroups still fit the 256 CUs at once
+// (43 column tiles: 4 or 5 slices 11.3 us, 6 slices = 258 workgroups 13.9 us; 112 tiles: 2 slices 39 us, 4 slices
+// 41 us), with at least two 32-row steps per wave (512 rows per 8-wave workgroup). `hint_parts` > 0 forces the count.
+inline void skinny_plan_one_round(int64_t k, int64_t n, int waves, int hint_parts, int *rows_per_block, int *splits, int *tiles) {
+    const int granule = 32 * waves;
+    const int64_t t = cdiv(n, kSkinnyTileN);
+    int64_t want = hint_parts;
+    if (want <= 0) want = std::min<int64_t>(std::max<int64_t>(1, 256 / t), std::max<int64_t>(1, k / (2 * granule)));
+    want = std::max<int64_t>(1, std::min<int64_t>(want, cdiv(k, granule)));
+    const int64_t rpb = cdiv(cdiv(k, want), granule) * granule;
+    *rows_per_block = int(rpb);
+    *splits = int(cdiv(k, rpb));
+    *tiles = int(t);
 }
 
-// Makes the plan fit the caller's workspace: fewer, longer K slices (down to one, which needs no workspace) when the
-// partial tiles would not fit. `strict` callers get an error instead, naming the bytes the plan needs.
-inline void skinny_fit_workspace(int64_t k, int granule, int tiles, int rows, const void *workspace, int64_t workspace_bytes,
-                                 bool strict, int *rows_per_block, int *splits) {
-    const int64_t avail = workspace != nullptr ? workspace_bytes : 0;
-    const int64_t need = skinny_workspace_need(tiles, *splits, rows);
-    if (need <= avail) return;
-    if (strict) QMM_FAIL("scratch too small for this shape: the K split needs " << need << " bytes, " << avail << " are there");
+// Bytes of mailbox a skinny launch with `splits` K slices touches: one fp32 partial tile per (column tile, K slice but
+// the last) of `rows` (at most 16) activation rows; the slot of the last slice is never written. One slice exchanges nothing.
+inline int64_t skinny_mailbox_need(int tiles, int splits, int rows) {
+    return splits > 1 ? int64_t(tiles) * splits * rows * kSkinnyTileN * 4 : 0;
+}
+
+// Makes the plan fit the mailbox: fewer, longer K slices (down to one, which needs none) when the partial tiles would
+// not fit. `strict` callers get an error instead, naming the bytes the plan needs.
+inline void skinny_fit_mailbox(int64_t k, int granule, int tiles, int rows, int64_t mailbox_bytes, bool strict,
+                               int *rows_per_block, int *splits) {
+    const int64_t need = skinny_mailbox_need(tiles, *splits, rows);
+    if (need <= mailbox_bytes) return;
+    if (strict) QMM_FAIL("scratch too small for this shape: the K split needs " << need << " bytes, " << mailbox_bytes << " are there");
     const int64_t per_split = int64_t(tiles) * rows * kSkinnyTileN * 4;
-    int64_t fit = avail > kCounterBytes ? (avail - kCounterBytes) / per_split : 1;
-    fit = std::max<int64_t>(1, std::min<int64_t>(fit, *splits));
+    int64_t fit = std::max<int64_t>(1, std::min<int64_t>(mailbox_bytes / per_split, *splits));
     const int64_t rpb = cdiv(cdiv(k, fit), granule) * granule;
     *rows_per_block = int(rpb);
     *splits = int(cdiv(k, rpb));

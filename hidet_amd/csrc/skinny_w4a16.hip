@@ -16,16 +16,16 @@
 namespace qmm {
 namespace {
 
+constexpr int kSkinnyWaves = 4;  // waves per workgroup; they split the workgroup's K slice
+
 template <int DT, int DEPTH, bool ALIGNED_A, bool FULL = false>
 __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,
                                                            const uint8_t *__restrict__ w,
                                                            const uint16_t *__restrict__ scales, uint16_t *__restrict__ c,
                                                            int m, int k, int n, int group, int rows_per_block, int splits,
-                                                           int tiles, float *__restrict__ partials,
-                                                           uint32_t *__restrict__ counters) {
+                                                           int tiles, float *__restrict__ mailbox) {
     using T = W4Traits<DT>;
     extern __shared__ float red[];
-    __shared__ int s_last;
 
     int tile, split;
     if (!skinny_tile_of_block(splits, tiles, &tile, &split)) return;
@@ -146,11 +146,11 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
             }
         }
     }
+    const SkinnyScale no_scale;  // all ones: the group scales are already in the totals
     if (DT == HIDET_QMM_F16)
-        skinny_reduce_store<_Float16>(total, m, n, tile, split, splits, nullptr, reinterpret_cast<_Float16 *>(c), partials,
-                                      counters, red, &s_last);
+        skinny_finish<_Float16, kSkinnyWaves>(total, m, n, tile, split, splits, no_scale, reinterpret_cast<_Float16 *>(c), mailbox, red);
     else
-        skinny_reduce_store<uint16_t>(total, m, n, tile, split, splits, nullptr, c, partials, counters, red, &s_last);
+        skinny_finish<uint16_t, kSkinnyWaves>(total, m, n, tile, split, splits, no_scale, c, mailbox, red);
 }
 
 // Any shape the fast kernel cannot take: one thread per output element, serial K, fp32 accumulation.
@@ -189,7 +189,7 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     const uint8_t *wp = static_cast<const uint8_t *>(w);
     const uint16_t *sp = static_cast<const uint16_t *>(scales);
     uint16_t *cp0 = static_cast<uint16_t *>(c);
-    if (!skinny_w4a16_fast(w, scales, k, n, group) || !aligned(c, 8)) {  // 8-byte output stores in the split-K sum
+    if (!skinny_w4a16_fast(w, scales, k, n, group)) {
         if (dtype == HIDET_QMM_F16)
             launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
         else
@@ -198,19 +198,17 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     }
     int rpb, splits, tiles;
     skinny_plan(k, n, 512, parallel_k_parts, 128, &rpb, &splits, &tiles);
-    QMM_CHECK(tiles <= kMaxSkinnyTiles, "N too large for the split-K counters");
-    skinny_fit_workspace(k, 128, tiles, int(std::min<int64_t>(16, m)), workspace, workspace_bytes, false, &rpb, &splits);
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
+    skinny_fit_mailbox(k, 128, tiles, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, &rpb, &splits);
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16);
     const int grid = int(cdiv(tiles, 8) * 8 * splits);
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
-        float *partials = reinterpret_cast<float *>(static_cast<char *>(workspace) + kCounterBytes);
-        uint32_t *counters = static_cast<uint32_t *>(workspace);
-        const size_t shmem = skinny_lds_bytes(mt);
+        const size_t shmem = skinny_lds_bytes(mt, kSkinnyWaves);
         auto go = [&](auto kern) {
-            if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16)));  // the most any m needs
+            if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16, kSkinnyWaves)));  // the most any m needs
             launch(kern, dim3(grid), dim3(256), shmem, stream, ap0 + m0 * lda, lda, wp, sp, cp0 + m0 * n, mt, int(k), int(n),
-                   group, rpb, splits, tiles, partials, counters);
+                   group, rpb, splits, tiles, ws.mailbox);
         };
         const bool full = aligned_a && n % kSkinnyTileN == 0 && k % rpb == 0 && rpb % (kSkinnyWaves * 64) == 0;
         if (full) {

@@ -58,7 +58,10 @@ static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_par
 // cover K exactly once, and every (column tile, slice) pair belongs to exactly one workgroup.
 static int check_skinny(long long k, long long ncols, int slice_rows, int hint, int granule) {
     int rpb = 0, splits = 0, tiles = 0;
-    skinny_plan(k, ncols, slice_rows, hint, granule, &rpb, &splits, &tiles);
+    if (slice_rows > 0) skinny_plan(k, ncols, slice_rows, hint, granule, &rpb, &splits, &tiles);
+    else skinny_plan_one_round(k, ncols, granule / 32, hint, &rpb, &splits, &tiles);  // the int8 kernel's plan
+    if (slice_rows == 0 && hint == 0 && (long long)(splits) * tiles > 256 && splits > 1)
+        return std::printf("skinny k=%lld n=%lld: %d slices x %d tiles do not fit one round\n", k, ncols, splits, tiles), 1;
     if (rpb <= 0 || rpb % granule != 0 || splits < 1 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
         tiles != int((ncols + kSkinnyTileN - 1) / kSkinnyTileN))
         return std::printf("skinny k=%lld n=%lld hint=%d: rows %d x %d splits, %d tiles\n", k, ncols, hint, rpb, splits, tiles), 1;
@@ -75,44 +78,52 @@ static int check_skinny(long long k, long long ncols, int slice_rows, int hint, 
     return 0;
 }
 
-// A plan cut down to a workspace: still whole granules covering K once, never more bytes than the workspace holds, the
+// A plan cut down to a mailbox: still whole granules covering K once, never more bytes than the mailbox holds, the
 // plan untouched when it fits, and a strict caller gets an error exactly when it does not.
-static int check_fit(long long k, long long ncols, int rows, long long workspace_bytes) {
+static int check_fit(long long k, long long ncols, int rows, long long workspace_bytes, int granule) {
     int rpb = 0, splits = 0, tiles = 0;
-    skinny_plan(k, ncols, rows > 8 ? 768 : 512, 0, 128, &rpb, &splits, &tiles);
+    if (granule == 256) skinny_plan_one_round(k, ncols, 8, 0, &rpb, &splits, &tiles);
+    else skinny_plan(k, ncols, rows > 8 ? 768 : 512, 0, granule, &rpb, &splits, &tiles);
     const int rpb0 = rpb, splits0 = splits;
-    char dummy = 0;
-    const bool fits = skinny_workspace_need(tiles, splits, rows) <= workspace_bytes;
+    static char dummy[16];
+    const Workspace ws = split_workspace(dummy, workspace_bytes);
+    if (workspace_bytes >= kCounterBytes &&
+        (ws.mailbox_bytes < 0 || ws.mailbox_bytes > kMaxMailboxBytes || ws.mailbox_bytes % 256 != 0 ||
+         kCounterBytes + ws.mailbox_bytes + ws.scratch_bytes != workspace_bytes ||
+         reinterpret_cast<char *>(ws.mailbox) + ws.mailbox_bytes != ws.scratch))
+        return std::printf("workspace of %lld bytes: mailbox %lld, scratch %lld\n", workspace_bytes, (long long)ws.mailbox_bytes, (long long)ws.scratch_bytes), 1;
+    const bool fits = skinny_mailbox_need(tiles, splits, rows) <= ws.mailbox_bytes;
     bool threw = false;
     try {
         int r2 = rpb, s2 = splits;
-        skinny_fit_workspace(k, 128, tiles, rows, &dummy, workspace_bytes, true, &r2, &s2);
+        skinny_fit_mailbox(k, granule, tiles, rows, ws.mailbox_bytes, true, &r2, &s2);
     } catch (const Error &) { threw = true; }
     if (threw == fits) return std::printf("fit k=%lld n=%lld rows=%d ws=%lld: strict error %d, fits %d\n", k, ncols, rows, workspace_bytes, threw, fits), 1;
-    skinny_fit_workspace(k, 128, tiles, rows, &dummy, workspace_bytes, false, &rpb, &splits);
+    skinny_fit_mailbox(k, granule, tiles, rows, ws.mailbox_bytes, false, &rpb, &splits);
     if (fits && (rpb != rpb0 || splits != splits0)) return std::printf("fit k=%lld n=%lld: a plan that fits was changed\n", k, ncols), 1;
-    if (rpb <= 0 || rpb % 128 != 0 || splits < 1 || splits > splits0 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
-        skinny_workspace_need(tiles, splits, rows) > workspace_bytes)
+    if (rpb <= 0 || rpb % granule != 0 || splits < 1 || splits > splits0 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
+        skinny_mailbox_need(tiles, splits, rows) > ws.mailbox_bytes)
         return std::printf("fit k=%lld n=%lld rows=%d ws=%lld: rows %d x %d splits need %lld\n", k, ncols, rows, workspace_bytes, rpb, splits,
-                           (long long)skinny_workspace_need(tiles, splits, rows)), 1;
+                           (long long)skinny_mailbox_need(tiles, splits, rows)), 1;
     return 0;
 }
 
 int main() {
     long long n = 0;
-    // 16384 x 128256 with 8 rows (an lm_head decode batch) wants 131 MB of partial tiles: it must come out within 64 MiB
-    for (long long ws : {0LL, 1024LL, 65536LL, 65536LL + 8192, 1LL << 20, 16LL << 20, (16LL << 20) + 65536, 64LL << 20})
+    // 16384 x 128256 with 8 rows (an lm_head decode batch) wants 131 MB of partial tiles: it must come out within the mailbox
+    for (long long ws : {0LL, 1024LL, 65536LL, 65536LL + 8192, 1LL << 20, 16LL << 20, (16LL << 20) + 65536, 64LL << 20, 96LL << 20})
         for (long long k : {128LL, 4096LL, 11008LL, 16384LL})
             for (long long nc : {256LL, 4096LL, 11008LL, 128256LL})
-                for (int rows : {1, 8, 16}) {
-                    if (check_fit(k, nc, rows, ws)) return 1;
-                    ++n;
-                }
+                for (int rows : {1, 8, 16})
+                    for (int granule : {128, 256, 512}) {
+                        if (check_fit(k, nc, rows, ws, granule)) return 1;
+                        ++n;
+                    }
     for (long long k : {32LL, 96LL, 128LL, 1000LL, 4096LL, 11008LL, 8192LL, 28672LL})
         for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL})
             for (int hint : {0, 1, 3, 8, 64})
-                for (int cfg = 0; cfg < 3; ++cfg) {
-                    if (check_skinny(k, nc, cfg == 1 ? 768 : 512, hint, cfg == 2 ? 256 : 128)) return 1;
+                for (int cfg = 0; cfg < 5; ++cfg) {
+                    if (check_skinny(k, nc, cfg == 1 ? 768 : cfg >= 3 ? 0 : 512, hint, cfg == 2 || cfg == 3 ? 256 : 128)) return 1;
                     ++n;
                 }
     const int cfgs[][3] = {{32, 32, 4}, {32, 32, 8}, {64, 64, 4}, {64, 32, 4}};  // concurrent, fill, max_parts of the launchers
