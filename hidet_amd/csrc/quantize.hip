@@ -87,7 +87,17 @@ __device__ __forceinline__ void load4_as_f32(const void *p, int64_t i4, float (&
     }
 }
 
-// code = saturating_cast(round_half_away(rnd(w / scale))), scale = rnd(amax / qmax), rnd = round to w's dtype.
+// code = saturating_cast(round(rnd(w / scale))), scale = rnd(amax / qmax), rnd = round to w's dtype. `round` is what
+// the reference's GPU lowering of round() does for the dtype: ties away from zero for float32 (roundf,
+// python/hidet/ir/primitives/hip/math/float32.py:40), ties to even for float16 (hrint, hip/math/float16.py:42) and
+// bfloat16 (hrint, cuda/math/bfloat16.py:29; the reference has no HIP bfloat16 math set). Its CPU half types round ties
+// away instead (include/hidet/runtime/cpu/float16.h:747-750): a float16 quotient of exactly n + 0.5 - common, since
+// float16 has a spacing of 1/16 between 64 and 128 - differs by one code between the two targets.
+template <int DT>
+__device__ __forceinline__ float round_code(float q) {
+    return DT == HIDET_QMM_F32 ? roundf(q) : rintf(q);
+}
+
 template <int DT, int QT>
 __global__ __launch_bounds__(256) void quantize_kernel(const void *__restrict__ w, const uint32_t *__restrict__ amax_bits,
                                                        void *__restrict__ q, void *__restrict__ scale, int64_t R,
@@ -102,7 +112,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(const void *__restrict__ 
     const float s = round_to<DT>(amax / qmax);
     if (r == 0) store_from_f32<DT>(scale, o * inner + c, s);
     float code = 0.0f;
-    if (s != 0.0f) code = roundf(round_to<DT>(load_as_f32<DT>(w, i) / s));
+    if (s != 0.0f) code = round_code<DT>(round_to<DT>(load_as_f32<DT>(w, i) / s));
     store_code<QT>(q, i, code);
 }
 
@@ -147,7 +157,7 @@ __global__ __launch_bounds__(256) void quantize4_kernel(const void *__restrict__
     for (int e = 0; e < 4; ++e) {
         const float s = round_to<DT>(__uint_as_float(abits[e]) / qmax);
         if (r == 0 && (!ALONG_REDUCE || e == 0)) store_from_f32<DT>(scale, sidx + (ALONG_REDUCE ? 0 : e), s);
-        code[e] = s != 0.0f ? roundf(round_to<DT>(x[e] / s)) : 0.0f;
+        code[e] = s != 0.0f ? round_code<DT>(round_to<DT>(x[e] / s)) : 0.0f;
     }
     if (QT == HIDET_QMM_I8) {
         uint32_t packed = 0;
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const void *__restri
         float x[4], code[4];
         load4_as_f32<DT>(w, i4, x);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) code[e] = s[e] != 0.0f ? roundf(round_to<DT>(x[e] / s[e])) : 0.0f;
+        for (int e = 0; e < 4; ++e) code[e] = s[e] != 0.0f ? round_code<DT>(round_to<DT>(x[e] / s[e])) : 0.0f;
         if (QT == HIDET_QMM_I8) {
             uint32_t packed = 0;
 #pragma unroll
@@ -243,7 +253,7 @@ __global__ __launch_bounds__(256) void quantize_row_fused_kernel(const void *__r
         if (j >= R4) continue;
         float code[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) code[e] = s != 0.0f ? roundf(round_to<DT>(x[v][e] / s)) : 0.0f;
+        for (int e = 0; e < 4; ++e) code[e] = s != 0.0f ? round_code<DT>(round_to<DT>(x[v][e] / s)) : 0.0f;
         if (QT == HIDET_QMM_I8) {
             uint32_t packed = 0;
 #pragma unroll

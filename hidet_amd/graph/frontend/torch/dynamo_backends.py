@@ -7,6 +7,7 @@ FlowGraph, optimizes it under a fresh PassContext and runs the compiled graph; w
 fresh context never does - and returns the rewritten GraphModule. Linear layers that meet the conditions of the fused
 rule run on the HIP W8A16 kernels; everything else stays on torch's own operators.
 """
+import copy
 from typing import Callable, List, Optional, Sequence
 
 import torch
@@ -52,9 +53,10 @@ def _cast_constants(gm: fx.GraphModule, dtype: torch.dtype) -> None:
                     setattr(mod, leaf, torch.nn.Parameter(cast, requires_grad=False))
                 else:
                     setattr(mod, leaf, cast)
-    for mod in gm.modules():
-        if mod is not gm:
-            mod.to(dtype)
+    # sub-modules the graph calls may be the caller's own objects: cast copies, never the originals
+    for name, child in list(gm.named_children()):
+        if any(t.dtype.is_floating_point and t.dtype != dtype for t in list(child.parameters()) + list(child.buffers())):
+            setattr(gm, name, copy.deepcopy(child).to(dtype))
 
 
 class CompiledModule:
@@ -107,6 +109,9 @@ def quantize_module(module: torch.nn.Module, ctx: Optional[PassContext] = None) 
     """Ahead-of-time form of the same rewrite: symbolic-trace `module`, cast its constants to the context's precision and
     apply the context's quantize rules. The result is an ordinary GraphModule (inputs are not cast for the caller)."""
     ctx = ctx if ctx is not None else PassContext.current()
+    # the rewrite casts and replaces constants: it works on a copy, the caller's module keeps its parameters and dtypes
+    # (the reference's from_torch leaves the torch model untouched as well)
+    module = copy.deepcopy(module)
     gm = module if isinstance(module, fx.GraphModule) else fx.symbolic_trace(module)
     precision = _PRECISIONS.get(ctx.configs['precision']) if ctx.configs['precision'] else None
     if precision is not None:

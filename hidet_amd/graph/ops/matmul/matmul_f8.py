@@ -59,19 +59,24 @@ class MatmulF8ScaledTask(Task):
 
 
 def _rows(x: torch.Tensor) -> torch.Tensor:
-    """2-D view whose last axis is contiguous (rows may be strided)."""
-    if x.stride(-1) != 1 and x.shape[-1] > 1:
+    """2-D operand the kernels can address as base + row * stride + column: the last axis contiguous and, with more
+    than one row, a row stride of at least the row length. Anything else (a transposed view, a row expanded with
+    stride 0, overlapping rows) is copied; rows that are merely strided are passed as they are."""
+    rows, cols = x.shape
+    if (cols > 1 and x.stride(1) != 1) or (rows > 1 and x.stride(0) < cols):
         x = x.contiguous()
     return x
+
+
+def _row_stride(x: torch.Tensor) -> int:
+    return x.stride(0) if x.shape[0] > 1 else x.shape[1]
 
 
 def _launch_f8(a2: torch.Tensor, b2: torch.Tensor, c2: torch.Tensor, scale_a, scale_b):
     m, k = a2.shape
     n = b2.shape[0]
-    lda = a2.stride(0) if m > 1 else k
-    ldb = b2.stride(0) if n > 1 else k
     ws = ffi.workspace(a2.device)
-    ffi.call('hidet_matmul_f8', a2, b2, c2, m, n, k, max(lda, k), max(ldb, k), ffi.DTYPE_CODE[c2.dtype], scale_a, scale_b,
+    ffi.call('hidet_matmul_f8', a2, b2, c2, m, n, k, _row_stride(a2), _row_stride(b2), ffi.DTYPE_CODE[c2.dtype], scale_a, scale_b,
              ws, ws.numel(), ffi.current_stream(a2.device))
 
 
@@ -121,20 +126,37 @@ class MatmulF8ScaledOperator(Operator):
             raise ValueError('only per-token (group_M = 1) x 128 x 128 block scaling is supported, got groups {}'.format((gm, gn, gk)))
         if scale_a.dtype != torch.float32 or scale_b.dtype != torch.float32:
             raise ValueError('scale_a and scale_b must be float32')
-        m, k = a.shape[-2], a.shape[-1]
-        n = b.shape[-2]
         out = self.attrs['output_dtype']
-        a3, b3 = a.reshape((-1, m, k)).contiguous(), b.reshape((-1, n, k)).contiguous()
-        sa3 = scale_a.reshape((-1,) + tuple(scale_a.shape[-2:])).contiguous()
-        sb3 = scale_b.reshape((-1,) + tuple(scale_b.shape[-2:])).contiguous()
-        if a3.shape[0] != b3.shape[0]:
-            raise ValueError('matmul_f8_scaled expects a and b with the same batch axes')
+        a3, b3, sa3, sb3, head = scaled_operands(a, b, scale_a, scale_b)
+        m, k = a3.shape[-2], a3.shape[-1]
+        n = b3.shape[-2]
         c = torch.empty((a3.shape[0], m, n), dtype=out, device=a.device)
         ws = ffi.workspace(a.device)
         for i in range(a3.shape[0]):
             ffi.call('hidet_matmul_f8_scaled', a3[i], b3[i], sa3[i], sb3[i], c[i], m, n, k, ffi.DTYPE_CODE[out],
                      ws, ws.numel(), ffi.current_stream(a.device))
-        return [c.reshape(tuple(a.shape[:-2]) + (m, n))]
+        return [c.reshape(head + (a.shape[-2], n))]
+
+
+def scaled_operands(a, b, scale_a, scale_b):
+    """Operands of the block-scaled matmul as dense 3-D tensors with one common batch axis, plus the head shape of the
+    result. The task accepts any mutually broadcastable heads (matmul_f8.py:372-376 of the reference): with a 2-D b
+    the batch axes of a are folded into M - scale_a [..., K/128, M] becomes [K/128, B * M] - and one launch serves
+    the whole batch; otherwise the heads are broadcast against each other."""
+    m, k = a.shape[-2], a.shape[-1]
+    n = b.shape[-2]
+    if b.dim() == 2 and a.dim() > 2:
+        head = tuple(a.shape[:-2])
+        a3 = a.reshape((1, -1, k)).contiguous()
+        kb = scale_a.shape[-2]
+        sa3 = scale_a.reshape((-1, kb, m)).permute(1, 0, 2).reshape((1, kb, -1)).contiguous()
+        return a3, b.reshape((1, n, k)).contiguous(), sa3, scale_b.reshape((1,) + tuple(scale_b.shape)).contiguous(), head
+    head = _broadcast_heads(a.shape[:-2], b.shape[:-2])
+    a3 = a.expand(head + (m, k)).reshape((-1, m, k)).contiguous()
+    b3 = b.expand(head + (n, k)).reshape((-1, n, k)).contiguous()
+    sa3 = scale_a.expand(head + tuple(scale_a.shape[-2:])).reshape((-1,) + tuple(scale_a.shape[-2:])).contiguous()
+    sb3 = scale_b.expand(head + tuple(scale_b.shape[-2:])).reshape((-1,) + tuple(scale_b.shape[-2:])).contiguous()
+    return a3, b3, sa3, sb3, head
 
 
 _VALIDATED = {}  # operand signature of an unscaled call that passed every check -> its output dtype

@@ -11,8 +11,8 @@ import torch
 from hidet_amd import option
 
 # The reference estimates 80 SMs x 5 resident blocks (resolve.py:46); an MI355X has 256 CUs and the
-# streaming kernel keeps about three workgroups resident on each.
-ESTIMATE_CONCURRENT_BLOCKS = 256 * 3
+# streaming kernel runs one round of one 8-wave workgroup on each.
+ESTIMATE_CONCURRENT_BLOCKS = 256
 SEARCH_CANDIDATES = [1, 2, 3, 4, 5, 6, 8, 10, 12, 16]  # resolve.py:54
 
 

@@ -15,9 +15,11 @@
  *     is explicit per call, so there is no global state besides the error string);
  *   - scratch memory comes from the caller as (workspace, workspace_bytes) instead of the
  *     reference's grow-only global request_hip_workspace (src/hidet/runtime/hip/context.cpp:43-57).
- *     The workspace must be zero-filled once when it is allocated; the kernels leave every counter
- *     they use at zero again.  Two calls that overlap in time (different streams) must not share
- *     a workspace.
+ *     The workspace must be zero-filled once when it is allocated.  Its first 64 KiB are arrival counters and the
+ *     next quarter of what remains (16 MiB at most) is the mailbox through which the bandwidth-bound kernels
+ *     exchange split-K partial sums: the kernels leave every counter and every mailbox word they use at zero
+ *     again.  The rest is plain scratch.  Two calls that overlap in time (different streams) must not share a
+ *     workspace, and nothing else may write to one while a call is in flight.
  *
  * All tensors are dense row-major.  No function allocates device memory or synchronises.
  */
@@ -75,8 +77,10 @@ void hidet_qmm_read_probe(const void *src, int64_t bytes, void *sink, void *stre
  * replaces the auto-scheduled kernels of SymmetricQuantizationTask / SymmetricDeQuantizationTask
  * (python/hidet/graph/ops/quant/symmetric.py:23-61).  The tensor is viewed as [outer, reduce, inner]
  * with the reduced axes folded into `reduce`; scale is [outer, inner] in w's dtype.
- *   scale = max|w| / qmax, wq = saturating_cast(round_half_away(w / scale)), evaluated in w's dtype
- *   (float32, float16 or bfloat16); a slice of zeros gives scale 0 and codes 0.
+ *   scale = max|w| / qmax, wq = saturating_cast(round(w / scale)), evaluated in w's dtype (float32, float16 or
+ *   bfloat16); round is the reference's GPU lowering for that dtype: ties away from zero for float32
+ *   (python/hidet/ir/primitives/hip/math/float32.py:40), ties to even for float16 and bfloat16
+ *   (hip/math/float16.py:42, cuda/math/bfloat16.py:29); a slice of zeros gives scale 0 and codes 0.
  * q_dtype is HIDET_QMM_I8 or HIDET_QMM_I16. */
 void hidet_symmetric_quantize(const void *w, void *wq, void *scale, int64_t outer, int64_t reduce, int64_t inner,
                               int w_dtype, int q_dtype, void *workspace, int64_t workspace_bytes, void *stream);
@@ -99,8 +103,8 @@ void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const voi
  * as hidet_symmetric_quant_matmul_f16_i8 called with a workspace of HIDET_QMM_STATIC_SCRATCH_BYTES; the scratch memory
  * is an array of that size inside the library's device code, one copy per GPU for the life of the process.  The call
  * allocates and frees nothing.  Up to 16 rows (and whenever the bandwidth-bound kernel is chosen) a shape whose K split
- * needs more partial-tile memory than the array holds is rejected with an error that names the bytes needed; taller
- * matrices always run, in as many K ranges as fit.  Every call on one GPU uses the same array: calls that overlap in
+ * needs more mailbox memory than the array's share of it (a quarter: 4 MiB) is rejected with an error that names the
+ * bytes needed; taller matrices always run, in as many K ranges as fit the scratch part.  Every call on one GPU uses the same array: calls that overlap in
  * time on one GPU (two streams, two threads) race; calls ordered by a stream or by events do not.  The device the
  * stream belongs to must be current. */
 #define HIDET_QMM_STATIC_SCRATCH_BYTES ((16 << 20) + (64 << 10))

@@ -119,8 +119,14 @@ def _normalize_dims(dims: Union[int, Sequence[int]], rank: int) -> Tuple[int, ..
 
 
 def symmetric_quantize(w: np.ndarray, quant_type: str = 'int8', dims: Union[int, Sequence[int]] = -1,
-                       dtype: Union[str, None] = None) -> Tuple[np.ndarray, np.ndarray]:
+                       dtype: Union[str, None] = None, target: str = 'cpu') -> Tuple[np.ndarray, np.ndarray]:
     """(wq, scale) of graph/ops/quant/symmetric.py:23-47,82-84.
+
+    `target` selects the reference's lowering of `round`, which depends on where the operator runs: 'cpu' rounds
+    ties away from zero for every dtype (roundf; include/hidet/runtime/cpu/float16.h:747-750, bfloat16.h:522-524),
+    'gpu' rounds ties away for float32 (ir/primitives/hip/math/float32.py:40) and ties to even for float16 and
+    bfloat16 (hrint: ir/primitives/hip/math/float16.py:42, cuda/math/float16.py:73, cuda/math/bfloat16.py:29). The HIP
+    kernels follow 'gpu'; the vectors recorded from the reference's CPU half type pin 'cpu'.
 
     `dims` are the reduced axes; `scale` has the remaining axes' shape.  All arithmetic is
     evaluated in the dtype of `w` (ir/dtypes/promotion.py:128-148): for float16/bfloat16 each of
@@ -145,7 +151,10 @@ def symmetric_quantize(w: np.ndarray, quant_type: str = 'int8', dims: Union[int,
     with np.errstate(divide='ignore', invalid='ignore'):
         quot = _round_to(w32 / scale32, dt).astype(np.float32)  # one division, rounded to w's dtype
     quot = np.where(scale32 == 0, np.float32(0), quot)
-    q = np.clip(round_half_away(quot), -qmax - 1, qmax).astype(INT_NP[quant_type])
+    if target not in ('cpu', 'gpu'):
+        raise ValueError("target must be 'cpu' or 'gpu', got {!r}".format(target))
+    rounded = np.rint(quot) if (target == 'gpu' and dt != 'float32') else round_half_away(quot)
+    q = np.clip(rounded, -qmax - 1, qmax).astype(INT_NP[quant_type])
     scale = _round_to(np.squeeze(scale32, axis=red), dt)
     return q, scale
 

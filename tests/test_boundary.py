@@ -178,3 +178,45 @@ def test_int4_decode_layout_repacking():
         assert np.array_equal((words >> np.uint32(4 * i)) & 0xF, u[kk].T)
     with pytest.raises(ValueError):
         to_decode_layout_int4(torch.zeros(12, 4, dtype=torch.uint8))
+
+
+def test_fp8_operand_normalisation():
+    # what reaches hidet_matmul_f8 must be addressable as base + row * stride + column with stride >= K: an expanded row
+    # (stride 0), a transposed view and overlapping rows are copied, a row-strided slice is passed through
+    from hidet_amd.graph.ops.matmul import matmul_f8 as F8
+    row = torch.arange(32, dtype=torch.uint8).view(1, 32)
+    exp = row.expand(5, 32)
+    got = F8._rows(exp)
+    assert got.stride() == (32, 1) and F8._row_stride(got) == 32 and torch.equal(got, exp)
+    wide = torch.arange(5 * 64, dtype=torch.uint8).view(5, 64)
+    sl = wide[:, 16:48]
+    assert F8._rows(sl).data_ptr() == sl.data_ptr() and F8._row_stride(F8._rows(sl)) == 64
+    tr = torch.arange(32 * 5, dtype=torch.uint8).view(32, 5).t()
+    assert F8._rows(tr).stride() == (32, 1) and torch.equal(F8._rows(tr), tr)
+    overlap = torch.arange(40, dtype=torch.uint8).as_strided((3, 32), (4, 1))
+    assert F8._rows(overlap).stride() == (32, 1) and torch.equal(F8._rows(overlap), overlap)
+    one = torch.arange(32, dtype=torch.uint8).as_strided((1, 32), (7, 1))
+    assert F8._row_stride(F8._rows(one)) == 32  # a single row: its stride is never used
+
+
+def test_fp8_scaled_operands_broadcast():
+    # batched activations against a 2-D weight fold into one launch: scale_a [B, K/128, M] -> [K/128, B * M]
+    from hidet_amd.graph.ops.matmul import matmul_f8 as F8
+    a = torch.arange(2 * 3 * 4 * 256, dtype=torch.float32).reshape(2, 3, 4, 256)
+    b = torch.arange(128 * 256, dtype=torch.float32).reshape(128, 256)
+    sa = torch.arange(2 * 3 * 2 * 4, dtype=torch.float32).reshape(2, 3, 2, 4)
+    sb = torch.arange(2, dtype=torch.float32).reshape(1, 2)
+    a3, b3, sa3, sb3, head = F8.scaled_operands(a, b, sa, sb)
+    assert head == (2, 3) and tuple(a3.shape) == (1, 24, 256) and tuple(b3.shape) == (1, 128, 256)
+    assert tuple(sa3.shape) == (1, 2, 24) and tuple(sb3.shape) == (1, 1, 2)
+    for bi in range(2):
+        for bj in range(3):
+            for r in range(4):
+                assert torch.equal(a3[0, (bi * 3 + bj) * 4 + r], a[bi, bj, r])
+                assert torch.equal(sa3[0, :, (bi * 3 + bj) * 4 + r], sa[bi, bj, :, r])
+    # heads that broadcast against each other
+    b5 = torch.zeros(3, 128, 256)
+    sb5 = torch.zeros(3, 1, 2)
+    a3, b3, sa3, sb3, head = F8.scaled_operands(a, b5, sa, sb5)
+    assert head == (2, 3) and a3.shape[0] == 6 and b3.shape[0] == 6 and sa3.shape[0] == 6 and sb3.shape[0] == 6
+    assert torch.equal(b3[4], b5[1]) and torch.equal(a3[4], a[1, 1])

@@ -225,6 +225,61 @@ def test_batched_and_strided_operands():
     assert np.array_equal(host(got).astype(np.int64), ai[0].astype(np.int64) @ bi.astype(np.int64).T)
 
 
+@pytest.mark.parametrize('m,k,n', [(6, 128, 16), (1, 1024, 512), (40, 512, 384), (300, 256, 520)])
+def test_per_tensor_exact_case(m, k, n):
+    # integer-valued codes and power-of-two scales: products, sums and the rescaling are exact in fp32
+    announce('fp8 per-tensor exact', m, k, n)
+    rng = np.random.default_rng(m + n)
+    ai, bi = rng.integers(-8, 9, (m, k)), rng.integers(-8, 9, (n, k))
+    ta, tb = f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32)))
+    for sa, sb in ((0.5, 4.0), (2.0 ** -6, 2.0 ** 3)):
+        want = (ai.astype(np.int64) @ bi.astype(np.int64).T).astype(np.float64) * sa * sb
+        dsa, dsb = dev(np.array([sa], dtype=np.float32)), dev(np.array([sb], dtype=np.float32))
+        got = F8.matmul_f8_per_tensor(ta, tb, dsa, dsb, 'float32')
+        assert np.array_equal(host(got).astype(np.float64), want)
+        gotb = F8.matmul_f8_per_tensor(ta, tb, dsa, dsb, 'bfloat16')
+        assert np.array_equal(host(gotb), O.to_bf16(want.astype(np.float32)))
+        assert np.array_equal(host(got), O.fp8_matmul_per_tensor(host(ta.view(torch.uint8)), host(tb.view(torch.uint8)),
+                                                                 np.float32(sa), np.float32(sb), 'float32'))
+
+
+def test_expanded_and_transposed_operands():
+    # operands whose rows cannot be addressed with a stride >= K (one row expanded to M rows, a transposed view) are
+    # copied by the operator before they reach the kernel
+    announce('fp8 expanded operands')
+    rng = np.random.default_rng(8)
+    row = rng.integers(-3, 3, (1, 256))
+    bi = rng.integers(-3, 3, (48, 256))
+    ta, tb = f8(O.e4m3_encode(row.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32)))
+    got = F8.matmul_f8(ta.expand(20, 256), tb, output_dtype='float32')
+    want = np.repeat(row.astype(np.int64), 20, axis=0) @ bi.astype(np.int64).T
+    assert np.array_equal(host(got).astype(np.int64), want)
+    at = rng.integers(-3, 3, (256, 24))
+    tt = f8(O.e4m3_encode(at.astype(np.float32)))
+    got = F8.matmul_f8(tt.t(), tb, output_dtype='float32')
+    assert np.array_equal(host(got).astype(np.int64), at.T.astype(np.int64) @ bi.astype(np.int64).T)
+    got = F8.matmul_f8(ta, tb.view(torch.uint8)[:1].expand(48, 256).view(torch.float8_e4m3fn), output_dtype='float32')
+    assert np.array_equal(host(got).astype(np.int64), row.astype(np.int64) @ np.repeat(bi[:1].astype(np.int64), 48, axis=0).T)
+
+
+def test_scaled_batched_activations_against_2d_weight():
+    # the task accepts mutually broadcastable heads (reference matmul_f8.py:372-376): [B, M, K] x [N, K]
+    announce('fp8 scaled batched')
+    rng = np.random.default_rng(9)
+    B, m, k, n = 3, 5, 256, 128
+    ai = rng.integers(-5, 5, (B, m, k))
+    bi = rng.integers(-5, 5, (n, k))
+    sa = rng.integers(1, 5, (B, k // 128, m)).astype(np.float32)
+    sb = rng.integers(1, 5, (n // 128, k // 128)).astype(np.float32)
+    got = F8.matmul_f8_scaled(f8(O.e4m3_encode(ai.astype(np.float32))), f8(O.e4m3_encode(bi.astype(np.float32))),
+                              scale_a=dev(sa), scale_b=dev(sb), output_dtype='float32')
+    assert tuple(got.shape) == (B, m, n)
+    b2 = bi.astype(np.int64) * np.repeat(np.repeat(sb.astype(np.int64), 128, axis=0), 128, axis=1)
+    for i in range(B):
+        a2 = ai[i].astype(np.int64) * np.repeat(sa[i].T.astype(np.int64), 128, axis=1)
+        assert np.array_equal(host(got[i]).astype(np.int64), a2 @ b2.T)
+
+
 def test_argument_errors():
     announce('fp8 errors')
     a = torch.zeros(4, 64, device='cuda').to(torch.float8_e4m3fn)

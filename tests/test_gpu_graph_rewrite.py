@@ -106,7 +106,7 @@ def test_ahead_of_time_rewrite_and_persisted_weights(tmp_path):
     assert O.max_rel_err(got.float().cpu().numpy(), want.cpu().numpy()) < 3e-2
     # the stored codes are what the oracle computes from the float16 weights, bit for bit
     w_kn = model.up.weight.detach().half().t().contiguous().cpu().numpy()
-    q, s = O.symmetric_quantize(w_kn, 'int8', dims=0)
+    q, s = O.symmetric_quantize(w_kn, 'int8', dims=0, target='gpu')
     assert np.array_equal(store['up.weight'][0].cpu().numpy(), q) and np.array_equal(store['up.weight'][1].cpu().numpy(), s)
     # save, load, rebuild from the stored weights only
     path = str(tmp_path / 'mlp_int8.npz')

@@ -39,12 +39,12 @@ def test_narrow_float_inputs_bit_exact(shape, dim, atype):
     if atype == 'float16':
         x = x32.astype(np.float16)
         tx = dev(x)
-        q0, s0 = O.symmetric_quantize(x, 'int8', dim)
+        q0, s0 = O.symmetric_quantize(x, 'int8', dim, target='gpu')
         s0b = s0.view(np.uint16)
     else:
         x = O.to_bf16(x32)
         tx = dev(x, torch.bfloat16)
-        q0, s0 = O.symmetric_quantize(x, 'int8', dim, dtype='bfloat16')
+        q0, s0 = O.symmetric_quantize(x, 'int8', dim, dtype='bfloat16', target='gpu')
         s0b = O.bf16_bits(s0)
     wq, scale = quant.symmetric_quantize(tx, dims=dim, quant_type='int8')
     assert np.array_equal(host(wq), q0)
@@ -65,9 +65,29 @@ def test_ties_zero_columns_and_saturation():
     assert np.array_equal(q[:, 2], -q[:, 0])
     # subnormal float16 scale: the quotient of the amax element reaches 128 and the cast saturates
     bits = np.array([0x0400, 0x8400, 0x0123, 0x0200], dtype=np.uint16).view(np.float16).reshape(-1, 1)
-    q0, s0 = O.symmetric_quantize(bits, 'int8', 0)
+    q0, s0 = O.symmetric_quantize(bits, 'int8', 0, target='gpu')
     wq, scale = quant.symmetric_quantize(dev(bits), 'int8', dims=0)
     assert np.array_equal(host(wq), q0) and np.array_equal(host(scale).view(np.uint16), s0.view(np.uint16))
+
+
+@pytest.mark.parametrize('atype', ['float16', 'bfloat16'])
+def test_narrow_float_ties_round_to_even(atype):
+    # the reference's GPU lowering of round() for float16 / bfloat16 is hrint (ties to even); float32 keeps roundf
+    # (ties away). amax 127 makes the scale exactly 1, so the quotients are the values themselves
+    announce('quantize ties to even', atype)
+    col = np.array([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, 64.5, -100.5, -101.5, 3.25, 3.75], dtype=np.float32)
+    want_even = [127, 0, 2, 2, 0, -2, -2, 64, 64, -100, -102, 3, 4]
+    want_away = [127, 1, 2, 3, -1, -2, -3, 64, 65, -101, -102, 3, 4]
+    w = np.stack([col, -col], axis=1)
+    tw = dev(w.astype(np.float16)) if atype == 'float16' else dev(O.to_bf16(w), torch.bfloat16)
+    wq, scale = quant.symmetric_quantize(tw, 'int8', dims=0)
+    assert host(wq)[:, 0].tolist() == want_even and host(wq)[:, 1].tolist() == [-v for v in want_even]
+    assert host(scale.float()).tolist() == [1.0, 1.0]
+    q_gpu, _ = O.symmetric_quantize(w, 'int8', 0, dtype=atype, target='gpu')
+    q_cpu, _ = O.symmetric_quantize(w, 'int8', 0, dtype=atype, target='cpu')
+    assert q_gpu[:, 0].tolist() == want_even and q_cpu[:, 0].tolist() == want_away
+    wq32, _ = quant.symmetric_quantize(dev(w), 'int8', dims=0)  # float32 input: ties away on every target
+    assert host(wq32)[:, 0].tolist() == want_away
 
 
 @pytest.mark.parametrize('shape,dims', [([4, 6, 10], [1]), ([4, 6, 10], [0, 2]), ([4, 6, 10], [0, 1, 2]), ([3, 5, 7, 2], [-1, -2]),
@@ -83,7 +103,7 @@ def test_general_dims(shape, dims):
     assert np.array_equal(_bits(host(back)), _bits(O.symmetric_dequantize(q0, s0, dims)))
 
 
-@pytest.mark.parametrize('k,n', [(4096, 4096), (4096, 11008), (11008, 4096)])
+@pytest.mark.parametrize('k,n', [(4096, 4096), (4096, 11008), (11008, 4096), (4096, 12288)])
 def test_benchmark_weight_shapes_bit_exact(k, n):
     announce('quantize benchmark shape', k, n)
     _, w = O.make_inputs(0, 1, k, n)
@@ -117,13 +137,13 @@ def test_one_scale_per_row_bit_exact(rows, cols, qt, atype):
     elif atype == 'float16':
         xh = x.astype(np.float16)
         t = dev(xh)
-        q0, s0 = O.symmetric_quantize(xh, qt, dims=-1)
+        q0, s0 = O.symmetric_quantize(xh, qt, dims=-1, target='gpu')
         s0b = s0.view(np.uint16)
         view = torch.int16
     else:
         xb = O.to_bf16(x)
         t = dev(xb, torch.bfloat16)
-        q0, s0 = O.symmetric_quantize(xb, qt, dims=-1, dtype='bfloat16')
+        q0, s0 = O.symmetric_quantize(xb, qt, dims=-1, dtype='bfloat16', target='gpu')
         s0b = O.bf16_bits(s0)
         view = torch.int16
     wq, scale = quant.symmetric_quantize(t, qt, dims=-1)

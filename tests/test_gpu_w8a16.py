@@ -60,7 +60,7 @@ def test_reference_recipe(x_shape, w_shape):
 
 @pytest.mark.parametrize('m,k,n,seed', [(16, 4096, 4096, 0), (1, 4096, 11008, 0), (1, 4096, 11008, 1),
                                         (1, 4096, 11008, 2), (1, 4096, 11008, 3), (1, 11008, 4096, 0),
-                                        (1, 11008, 4096, 3), (5, 1000, 528, 0), (33, 512, 256, 0), (13, 4096, 11008, 0)])
+                                        (1, 11008, 4096, 1), (1, 11008, 4096, 2), (1, 11008, 4096, 3), (5, 1000, 528, 0), (33, 512, 256, 0), (13, 4096, 11008, 0)])
 def test_parity_with_oracle(m, k, n, seed):
     announce('w8a16 parity', m, k, n, seed)
     a, q, s = _case(seed, m, k, n)
@@ -97,6 +97,26 @@ def test_split_k_parts_api_and_hints():
         finally:
             hidet_amd.option.parallel_k('disabled')
         assert O.max_rel_err(host(c), host(base)) < 1e-3
+
+
+def test_parallel_k_search():
+    # hidet.option.parallel_k('search') (reference resolve.py:53-92): the candidates are timed on the GPU, the winner is
+    # one of them (or 0, the library's own plan), is remembered per shape, and the result equals the unsplit one
+    from hidet_amd.graph.ops.quant import resolve
+    announce('w8a16 parallel_k search')
+    a, q, s = _int_case(11, 2, 1024, 512)
+    ta, tq, ts = dev(a), dev(q), dev(s)
+    want = host(quant.symmetric_quant_matmul(ta, tq, ts))
+    resolve._SEARCH_CACHE.clear()
+    hidet_amd.option.parallel_k('search')
+    try:
+        got = host(quant.symmetric_quant_matmul(ta, tq, ts))
+        hint = resolve.resolve_parallel_k_parts('search', ta, tq)
+    finally:
+        hidet_amd.option.parallel_k('disabled')
+    assert hint in [0] + resolve.SEARCH_CANDIDATES
+    assert resolve._SEARCH_CACHE == {((2, 1024), (1024, 512)): hint}
+    assert np.array_equal(got, want)  # small integers: exact whatever the split
 
 
 def test_deterministic_and_counters_reset():

@@ -107,6 +107,21 @@ def test_linear_modules_become_fused_operator(cpu_ops):
     assert O.max_rel_err(got.float().numpy(), want.detach().numpy()) < 3e-2
 
 
+def test_quantize_module_leaves_the_source_model_untouched(cpu_ops):
+    # the rewrite casts constants to float16 and swaps weights for int8 codes in a copy; the caller's model keeps its
+    # float32 parameters, bit for bit
+    torch.manual_seed(4)
+    model = Mlp().eval()
+    before = {k: v.clone() for k, v in model.state_dict().items()}
+    with PassContext() as ctx:
+        ctx.set_precision('int8')
+        quantize_module(model, ctx)
+    after = model.state_dict()
+    assert set(after) == set(before)
+    for k, v in before.items():
+        assert after[k].dtype == torch.float32 and torch.equal(after[k], v), k
+
+
 def test_decode_layout_keeps_codes_k_contiguous_and_releases_the_rest(cpu_ops):
     torch.manual_seed(2)
     model = Mlp().eval()

@@ -135,6 +135,29 @@ def test_symmetric_quantize_constructed_ties_round_away():
     assert qc[:, 0].tolist() == q[:, 0].tolist()
 
 
+@pytest.mark.parametrize('dtype', ['float16', 'bfloat16'])
+def test_symmetric_quantize_tie_rule_per_target(dtype):
+    # the reference lowers round() per target: ties away on the CPU for every dtype, ties to even (hrint) on the GPU for
+    # float16 / bfloat16, ties away (roundf) on the GPU for float32. Scale is exactly 1 here.
+    col = np.array([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, 64.5, -100.5, -101.5, 3.25, 3.75], dtype=np.float32)
+    away = [127, 1, 2, 3, -1, -2, -3, 64, 65, -101, -102, 3, 4]
+    even = [127, 0, 2, 2, 0, -2, -2, 64, 64, -100, -102, 3, 4]
+    q_cpu, s = O.symmetric_quantize(col[:, None], 'int8', 0, dtype=dtype, target='cpu')
+    q_gpu, _ = O.symmetric_quantize(col[:, None], 'int8', 0, dtype=dtype, target='gpu')
+    assert float(s[0]) == 1.0 and q_cpu[:, 0].tolist() == away and q_gpu[:, 0].tolist() == even
+    q32_cpu, _ = O.symmetric_quantize(col[:, None], 'int8', 0, target='cpu')
+    q32_gpu, _ = O.symmetric_quantize(col[:, None], 'int8', 0, target='gpu')
+    assert q32_cpu[:, 0].tolist() == away and q32_gpu[:, 0].tolist() == away
+    # away from exact ties the two targets agree
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((64, 8)).astype(np.float32)
+    qa, _ = O.symmetric_quantize(x, 'int8', 0, dtype=dtype, target='cpu')
+    qb, _ = O.symmetric_quantize(x, 'int8', 0, dtype=dtype, target='gpu')
+    assert np.abs(qa.astype(np.int32) - qb.astype(np.int32)).max() <= 1
+    with pytest.raises(ValueError):
+        O.symmetric_quantize(x, 'int8', 0, target='tpu')
+
+
 @pytest.mark.skipif(clib.ref_lib() is None, reason='oracle/_ref not built (reference checkout absent)')
 def test_symmetric_quantize_f16_brute_force_against_reference_half_type():
     # every finite positive float16 pattern in one column (the largest value fixes the scale),
@@ -312,9 +335,25 @@ def test_group_quantize_int4_invariants():
     g = np.abs(q.astype(np.int32)).reshape(4, 128, 64).max(axis=1)
     assert np.all(g[amax > 0] == 7) and np.all(g[amax == 0] == 0) and np.abs(q).max() <= 7
     assert np.array_equal(O.unpack_int4(packed), q)
-    # dequantized weights stay within half a step (plus bf16 rounding of the scale) of the original
-    wd = np.repeat(scales, 128, axis=0) * q
-    assert np.max(np.abs(wd - w)) <= np.max(scales) * 0.51
+    # dequantized weights stay within half a step of their own group's scale of the original, plus the bf16 rounding of
+    # that scale (relative 2^-8 at most) on codes of magnitude 7 at most
+    step = np.repeat(scales, 128, axis=0)
+    assert np.all(np.abs(step * q - w) <= step * (0.5 + 7 * 2.0 ** -8) * (1 + 2.0 ** -8))
+
+
+def test_group_quantize_int4_constructed_ties_and_clamp():
+    # a group whose amax is 7 has scale32 exactly 1: the codes are round_half_away of the values themselves
+    col = np.zeros(128, dtype=np.float32)
+    vals = np.array([7.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 6.5, -6.5, 3.49, -3.51], dtype=np.float32)
+    col[:vals.size] = vals
+    w = np.stack([col, -col, 2 * col], axis=1).astype(np.float32)
+    w = np.concatenate([w, w[:, :1]], axis=1)  # an even number of columns
+    packed, scales, q = O.group_quantize_int4(w, 128, 'float16')
+    want = [7, 1, 2, 3, -1, -2, -3, 7, -7, 3, -4]
+    assert q[:vals.size, 0].tolist() == want and q[:vals.size, 1].tolist() == [-v for v in want]
+    assert q[:vals.size, 2].tolist() == want  # scale 2: the same quotients
+    assert scales[0].astype(np.float32).tolist() == [1.0, 1.0, 2.0, 1.0]
+    assert np.array_equal(O.unpack_int4(packed), q)
 
 
 def test_w4a16_matmul_exact_on_small_integers():
@@ -421,6 +460,26 @@ def test_fp8_per_tensor_quantize_and_matmul():
     assert O.max_rel_err(out, ref) < 5e-3  # only the bf16 output rounding remains
     zc, zs = O.fp8_quantize_per_tensor(np.zeros((2, 2), dtype=np.float32))
     assert zs == 0 and not zc.any()
+
+
+def test_fp8_per_tensor_matmul_exact_case():
+    # integer-valued e4m3 codes and power-of-two scales: every product, the sum and the rescaling are exact in fp32,
+    # so a dropped scale, a transposed operand or a wrong accumulation shows as a whole-number difference
+    rng = np.random.default_rng(17)
+    ai = rng.integers(-8, 9, (6, 128))
+    bi = rng.integers(-8, 9, (10, 128))
+    ac, bc = O.e4m3_encode(ai.astype(np.float32)), O.e4m3_encode(bi.astype(np.float32))
+    assert np.array_equal(O.e4m3_decode(ac), ai) and np.array_equal(O.e4m3_decode(bc), bi)
+    for sa, sb in ((0.5, 4.0), (2.0 ** -6, 2.0 ** 3), (1.0, 1.0)):
+        want = (ai.astype(np.int64) @ bi.astype(np.int64).T).astype(np.float64) * sa * sb
+        got = O.fp8_matmul_per_tensor(ac, bc, np.float32(sa), np.float32(sb), 'float32')
+        assert np.array_equal(got.astype(np.float64), want)
+        gotb = O.fp8_matmul_per_tensor(ac, bc, np.float32(sa), np.float32(sb), 'bfloat16')
+        assert np.array_equal(gotb, O.to_bf16(want.astype(np.float32)))
+    # per-tensor quantization of a tensor whose amax is 448 * 2^j leaves every representable value unchanged
+    x = np.array([[448.0, -3.0, 0.25, 9.0 / 8.0]], dtype=np.float32) * np.float32(4.0)
+    codes, scale = O.fp8_quantize_per_tensor(x)
+    assert scale == np.float32(4.0) and np.array_equal(O.e4m3_decode(codes) * scale, x)
 
 
 def test_max_rel_err_definition():

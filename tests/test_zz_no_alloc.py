@@ -84,7 +84,8 @@ def test_static_scratch_exact_on_small_integers():
 
 
 def test_static_scratch_rejects_oversized_split():
-    # 16 rows, K = 16384, N = 32768: 128 column tiles x 21 K slices x 16 KiB of partial tiles = 43 MB > 16 MiB
+    # 16 rows, K = 16384, N = 32768, 16 K slices asked for: 128 column tiles x 16 slices x 16 KiB of partial tiles = 32 MiB,
+    # more than the mailbox share (4 MiB) of the static array
     m, k, n = 16, 16384, 32768
     announce('static scratch reject', m, k, n)
     a = torch.zeros((m, k), dtype=torch.float16, device='cuda')
