@@ -10,6 +10,10 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
                      hipStream_t stream);
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
                             int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+void skinny_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                            int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
+void gemm_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                          int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
 void skinny_fp8_block_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
                                     int64_t n, int64_t k, int out_dtype, hipStream_t stream);
 }  // namespace qmm
@@ -44,6 +48,24 @@ HIDET_API void hidet_matmul_f8(const void *a, const void *b, void *c, int64_t m,
         skinny_fp8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
     else
         gemm_fp8_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, workspace, workspace_bytes, stream);
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_matmul_f8_e5m2(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda,
+                                    int64_t ldb, int out_dtype, const void *scale_a, const void *scale_b, void *stream_) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(out_dtype == HIDET_QMM_F32 || out_dtype == HIDET_QMM_F16 || out_dtype == HIDET_QMM_BF16 || out_dtype == HIDET_QMM_E5M2,
+              "output dtype must be float32, float16, bfloat16 or float8_e5m2, got code " << out_dtype);
+    QMM_CHECK(m >= 0 && n >= 0 && k >= 0, "negative extent: m=" << m << " n=" << n << " k=" << k);
+    QMM_CHECK(lda >= k && ldb >= k, "row strides (" << lda << ", " << ldb << ") must be at least K (" << k << ")");
+    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    if (m == 0 || n == 0) return;
+    QMM_CHECK(c && (k == 0 || (a && b)), "null tensor pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (m <= 16 && skinny_fp8_supported(b, k, ldb))
+        skinny_fp8_e5m2_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
+    else
+        gemm_fp8_e5m2_launch(a, b, c, m, n, k, lda, ldb, out_dtype, scale_a, scale_b, stream);
     QMM_ENTRY_END
 }
 

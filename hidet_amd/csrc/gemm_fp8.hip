@@ -22,14 +22,15 @@ constexpr int kStageChunks = (kBM + kBN) * 8;      // 16-byte chunks per stage (
 constexpr int kChunksPerThread = kStageChunks / kThreads;  // 16
 constexpr int kLdsBytes = 2 * kStageChunks * 16;   // 128 KiB
 
+template <int FMT = kFmtE4M3>
 __device__ __forceinline__ float4_t mfma_fp8_k128(const uint4 &r0, const uint4 &r1, const uint4 &c0, const uint4 &c1, float4_t acc) {
     int8v_t rv, cv;
     rv[0] = int(r0.x); rv[1] = int(r0.y); rv[2] = int(r0.z); rv[3] = int(r0.w);
     rv[4] = int(r1.x); rv[5] = int(r1.y); rv[6] = int(r1.z); rv[7] = int(r1.w);
     cv[0] = int(c0.x); cv[1] = int(c0.y); cv[2] = int(c0.z); cv[3] = int(c0.w);
     cv[4] = int(c1.x); cv[5] = int(c1.y); cv[6] = int(c1.z); cv[7] = int(c1.w);
-    // formats 0/0 = e4m3 x e4m3; block scales 0x7F = 2^0
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    // formats FMT / FMT: 0 = e4m3, 1 = e5m2 for both operands; block scales 0x7F = 2^0
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
 
 template <int OUT>
@@ -46,6 +47,10 @@ __device__ __forceinline__ void store4(void *c, int64_t idx, float4_t v) {
         o.x = uint32_t(f32_to_f16_bits(v[0])) | (uint32_t(f32_to_f16_bits(v[1])) << 16);
         o.y = uint32_t(f32_to_f16_bits(v[2])) | (uint32_t(f32_to_f16_bits(v[3])) << 16);
         *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + idx) = o;
+    } else if (OUT == HIDET_QMM_E5M2) {
+        const uint32_t o = uint32_t(f32_to_e5m2(v[0])) | (uint32_t(f32_to_e5m2(v[1])) << 8) |
+                           (uint32_t(f32_to_e5m2(v[2])) << 16) | (uint32_t(f32_to_e5m2(v[3])) << 24);
+        *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(c) + idx) = o;
     } else {
         const uint32_t o = uint32_t(f32_to_e4m3(v[0])) | (uint32_t(f32_to_e4m3(v[1])) << 8) |
                            (uint32_t(f32_to_e4m3(v[2])) << 16) | (uint32_t(f32_to_e4m3(v[3])) << 24);
@@ -53,7 +58,7 @@ __device__ __forceinline__ void store4(void *c, int64_t idx, float4_t v) {
     }
 }
 
-template <int OUT>
+template <int OUT, int FMT = kFmtE4M3>
 __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_staged_kernel(const uint8_t *__restrict__ a, int64_t lda,
                                                                const uint8_t *__restrict__ b, int64_t ldb,
                                                                void *__restrict__ c, int m, int n, int k,
@@ -125,7 +130,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_staged_kernel(const uint
             const uint4 a0 = la[r * 8 + ((2 * kg) ^ (r & 7))];
             const uint4 a1 = la[r * 8 + ((2 * kg + 1) ^ (r & 7))];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) acc[i][j] = mfma_fp8_k128(bf[j][0], bf[j][1], a0, a1, acc[i][j]);
+            for (int j = 0; j < 8; ++j) acc[i][j] = mfma_fp8_k128<FMT>(bf[j][0], bf[j][1], a0, a1, acc[i][j]);
         }
         if (more) store_stage(buf ^ 1);
         __syncthreads();
@@ -394,7 +399,7 @@ __global__ __launch_bounds__(WAVES * 64, 1) void gemm_fp8_kernel(const uint8_t *
 }
 
 // Fallback for shapes the tiled kernel cannot take: one thread per output element.
-template <int OUT>
+template <int OUT, int FMT = kFmtE4M3>
 __global__ __launch_bounds__(256) void naive_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ b,
                                                         int64_t ldb, void *__restrict__ c, int64_t m, int64_t n, int64_t k,
                                                         const float *__restrict__ scale_a, const float *__restrict__ scale_b) {
@@ -402,13 +407,10 @@ __global__ __launch_bounds__(256) void naive_fp8_kernel(const uint8_t *__restric
     if (o >= m * n) return;
     const int64_t i = o / n, j = o - i * n;
     float acc = 0.f;
-    for (int64_t kk = 0; kk < k; ++kk) acc += e4m3_to_f32(a[i * lda + kk]) * e4m3_to_f32(b[j * ldb + kk]);
+    for (int64_t kk = 0; kk < k; ++kk) acc += fp8_to_f32<FMT>(a[i * lda + kk]) * fp8_to_f32<FMT>(b[j * ldb + kk]);
     if (scale_a != nullptr) acc *= (*scale_a) * (scale_b != nullptr ? *scale_b : 1.0f);
     else if (scale_b != nullptr) acc *= *scale_b;
-    if (OUT == HIDET_QMM_F32) static_cast<float *>(c)[o] = acc;
-    else if (OUT == HIDET_QMM_BF16) static_cast<uint16_t *>(c)[o] = f32_to_bf16_bits(acc);
-    else if (OUT == HIDET_QMM_F16) static_cast<uint16_t *>(c)[o] = f32_to_f16_bits(acc);
-    else static_cast<uint8_t *>(c)[o] = f32_to_e4m3(acc);
+    store_out<OUT>(c, o, acc);
 }
 
 template <typename F>
@@ -422,7 +424,41 @@ void dispatch_out(int out_dtype, F &&f) {
     }
 }
 
+// float8_e5m2 operands: the register-staged tile kernel with the MFMA's bf8 format, or the element-wise kernel
+template <typename F>
+void dispatch_out_e5m2(int out_dtype, F &&f) {
+    switch (out_dtype) {
+        case HIDET_QMM_F32: f(std::integral_constant<int, HIDET_QMM_F32>()); break;
+        case HIDET_QMM_F16: f(std::integral_constant<int, HIDET_QMM_F16>()); break;
+        case HIDET_QMM_BF16: f(std::integral_constant<int, HIDET_QMM_BF16>()); break;
+        case HIDET_QMM_E5M2: f(std::integral_constant<int, HIDET_QMM_E5M2>()); break;
+        default: QMM_FAIL("unsupported output dtype code " << out_dtype << " for float8_e5m2 operands");
+    }
+}
+
 }  // namespace
+
+void gemm_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                          int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
+    const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
+    const float *sa = static_cast<const float *>(scale_a), *sb = static_cast<const float *>(scale_b);
+    const bool tiled = (k % 16 == 0) && (lda % 16 == 0) && (ldb % 16 == 0) && (n % 4 == 0) && aligned(a, 16) &&
+                       aligned(b, 16) && aligned(c, 16) && k > 0;
+    dispatch_out_e5m2(out_dtype, [&](auto o) {
+        constexpr int OUT = decltype(o)::value;
+        if (!tiled) {
+            launch(naive_fp8_kernel<OUT, kFmtE5M2>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap, lda, bp, ldb, c, m, n, k, sa, sb);
+            return;
+        }
+        const int tiles_m = int(cdiv(m, kBM)), tiles_n = int(cdiv(n, kBN));
+        const GemmTiling tiling = make_gemm_tiling(tiles_m, tiles_n, 32);
+        const int64_t grid = tiling.grid();
+        QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
+        allow_dynamic_lds(reinterpret_cast<const void *>(gemm_fp8_staged_kernel<OUT, kFmtE5M2>), kLdsBytes);
+        launch(gemm_fp8_staged_kernel<OUT, kFmtE5M2>, dim3(uint32_t(grid)), dim3(kThreads), size_t(kLdsBytes), stream, ap, lda, bp,
+               ldb, c, int(m), int(n), int(k), sa, sb, tiles_m, tiles_n, tiling.xm, tiling.xn);
+    });
+}
 
 void gemm_fp8_kernel8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
                              int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,

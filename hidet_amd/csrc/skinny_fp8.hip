@@ -16,7 +16,7 @@ constexpr int kWaves = 4;
 constexpr int kEightWaveTiles = 512;  // fewer column tiles than this: eight waves per workgroup (8192 x 4096: 9.4 -> 7.2 us)
 constexpr int kDepth = 8;  // k-steps (of 128 bytes) whose loads are issued together
 
-template <int OUT, bool ALIGNED_A>
+template <int OUT, bool ALIGNED_A, int FMT = kFmtE4M3>
 __global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restrict__ a, int64_t lda,
                                                          const uint8_t *__restrict__ b, int64_t ldb, void *__restrict__ c,
                                                          int m, int n, int k, const float *__restrict__ scale_a,
@@ -78,8 +78,8 @@ __global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restri
             rv[4] = int(xv[d][1].x); rv[5] = int(xv[d][1].y); rv[6] = int(xv[d][1].z); rv[7] = int(xv[d][1].w);
             cv[0] = int(wv[d][0].x); cv[1] = int(wv[d][0].y); cv[2] = int(wv[d][0].z); cv[3] = int(wv[d][0].w);
             cv[4] = int(wv[d][1].x); cv[5] = int(wv[d][1].y); cv[6] = int(wv[d][1].z); cv[7] = int(wv[d][1].w);
-            // rows = activation rows, columns = rows of b; formats e4m3 x e4m3, unit block scales
-            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+            // rows = activation rows, columns = rows of b; both operands in format FMT, unit block scales
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
         }
     }
     // acc[v] = partial c[4 kg + v][n0 + ls]
@@ -91,11 +91,7 @@ __global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restri
         float v = red[0][row][cn] + red[1][row][cn] + red[2][row][cn] + red[3][row][cn];
         if (scale_a != nullptr) v *= *scale_a;
         if (scale_b != nullptr) v *= *scale_b;
-        const int64_t o = int64_t(row) * n + n0 + cn;
-        if (OUT == HIDET_QMM_F32) static_cast<float *>(c)[o] = v;
-        else if (OUT == HIDET_QMM_BF16) static_cast<uint16_t *>(c)[o] = f32_to_bf16_bits(v);
-        else if (OUT == HIDET_QMM_F16) static_cast<uint16_t *>(c)[o] = f32_to_f16_bits(v);
-        else static_cast<uint8_t *>(c)[o] = f32_to_e4m3(v);
+        store_out<OUT>(c, int64_t(row) * n + n0 + cn, v);
     }
 }
 
@@ -226,6 +222,27 @@ void skinny_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t
         default: QMM_FAIL("unsupported output dtype code " << out_dtype);
     }
 #undef QMM_FP8_SKINNY
+}
+
+// float8_e5m2 operands, up to 16 rows: the plain kernel with the MFMA's bf8 format
+void skinny_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                            int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream) {
+    const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
+    const float *sa = static_cast<const float *>(scale_a), *sb = static_cast<const float *>(scale_b);
+    const bool aligned_a = (lda % 16 == 0) && aligned(a, 16);
+    const dim3 grid(uint32_t(cdiv(n, 16)));
+    auto go = [&](auto kern) { launch(kern, grid, dim3(256), 0, stream, ap, lda, bp, ldb, c, int(m), int(n), int(k), sa, sb); };
+#define QMM_BF8_SKINNY(OUT)                                           \
+    if (aligned_a) go(skinny_fp8_kernel<OUT, true, kFmtE5M2>);        \
+    else go(skinny_fp8_kernel<OUT, false, kFmtE5M2>);
+    switch (out_dtype) {
+        case HIDET_QMM_F32: QMM_BF8_SKINNY(HIDET_QMM_F32) break;
+        case HIDET_QMM_F16: QMM_BF8_SKINNY(HIDET_QMM_F16) break;
+        case HIDET_QMM_BF16: QMM_BF8_SKINNY(HIDET_QMM_BF16) break;
+        case HIDET_QMM_E5M2: QMM_BF8_SKINNY(HIDET_QMM_E5M2) break;
+        default: QMM_FAIL("unsupported output dtype code " << out_dtype << " for float8_e5m2 operands");
+    }
+#undef QMM_BF8_SKINNY
 }
 
 // Block-scaled operands (scale_a f32 [K/128, M], scale_b f32 [N/128, K/128]), up to 16 rows, contiguous a [M, K] and b [N, K],

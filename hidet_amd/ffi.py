@@ -18,10 +18,10 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libhidet_qmm.so')
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 
 # dtype codes of include/hidet_qmm.h
-F32, F16, BF16, I8, I16, E4M3 = 0, 1, 2, 3, 4, 5
+F32, F16, BF16, I8, I16, E4M3, E5M2 = 0, 1, 2, 3, 4, 5, 6
 DTYPE_CODE = {
     torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.int8: I8, torch.int16: I16,
-    torch.float8_e4m3fn: E4M3,
+    torch.float8_e4m3fn: E4M3, torch.float8_e5m2: E5M2,
 }
 
 # name -> (restype, argtypes): every symbol include/hidet_qmm.h declares
@@ -49,6 +49,7 @@ SIGNATURES = {
     'hidet_symmetric_quant_matmul_w4a16_nk': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _vp]),
     'hidet_fp8_quantize_per_tensor': (None, [_vp, _vp, _vp, _i64, _i32, _vp, _i64, _vp]),
     'hidet_matmul_f8': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _i64, _vp]),
+    'hidet_matmul_f8_e5m2': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp]),
     'hidet_matmul_f8_scaled': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
 }
 

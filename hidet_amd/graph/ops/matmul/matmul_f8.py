@@ -2,8 +2,9 @@
 (python/hidet/graph/ops/matmul/matmul_f8.py:132-175, 357-454, 644-775), executed by `hidet_matmul_f8` and
 `hidet_matmul_f8_scaled`, plus the per-tensor quantize / matmul pair of the benchmark configuration.
 
-A is [..., M, K] and B is [..., N, K], both K-major.  Only float8_e4m3 is built (the MI355X native OCP
-format); float8_e5m2 operands are rejected with an explicit error."""
+A is [..., M, K] and B is [..., N, K], both K-major, both float8_e4m3 or both float8_e5m2 (OCP formats, the MFMA's
+fp8 and bf8 operand types).  The e4m3 path has the tuned kernels; e5m2 runs the unscaled matmul on plainer ones, and
+the block-scaled matmul is built for e4m3 only."""
 from typing import List, Optional, Tuple
 
 import torch
@@ -13,7 +14,7 @@ from hidet_amd.graph.operator import Operator, Task, TensorSpec, data_type, inpu
 
 f8e4m3 = torch.float8_e4m3fn
 f8e5m2 = torch.float8_e5m2
-_OUT_TYPES = (torch.float32, torch.float16, torch.bfloat16, f8e4m3)
+_OUT_TYPES = (torch.float32, torch.float16, torch.bfloat16, f8e4m3, f8e5m2)
 
 
 def _broadcast_heads(a_head, b_head) -> Tuple[int, ...]:
@@ -75,6 +76,10 @@ def _row_stride(x: torch.Tensor) -> int:
 def _launch_f8(a2: torch.Tensor, b2: torch.Tensor, c2: torch.Tensor, scale_a, scale_b):
     m, k = a2.shape
     n = b2.shape[0]
+    if a2.dtype == f8e5m2:  # the bf8 format of the MFMA, on the plainer kernels (no workspace)
+        ffi.call('hidet_matmul_f8_e5m2', a2, b2, c2, m, n, k, _row_stride(a2), _row_stride(b2), ffi.DTYPE_CODE[c2.dtype],
+                 scale_a, scale_b, ffi.current_stream(a2.device))
+        return
     ws = ffi.workspace(a2.device)
     ffi.call('hidet_matmul_f8', a2, b2, c2, m, n, k, _row_stride(a2), _row_stride(b2), ffi.DTYPE_CODE[c2.dtype], scale_a, scale_b,
              ws, ws.numel(), ffi.current_stream(a2.device))
@@ -171,16 +176,16 @@ def _matmul_f8(a, b, is_scaled: bool, scale_a=None, scale_b=None, bias=None, acc
         raise ValueError('a and b must have at least 2 dimensions, got shape {} and {}'.format(list(a.shape), list(b.shape)))
     if (a.dtype != f8e4m3 or b.dtype != f8e4m3) and (a.dtype != f8e5m2 or b.dtype != f8e5m2):
         raise ValueError('matmul_f8 only supports both operands being f8e4m3 or f8e5m2, got {} and {}'.format(a.dtype, b.dtype))
-    if a.dtype == f8e5m2:
-        raise NotImplementedError('float8_e5m2 operands are not built in this library: only float8_e4m3 kernels exist')
+    if a.dtype == f8e5m2 and is_scaled:
+        raise NotImplementedError('block-scaled matmul is built for float8_e4m3 operands only')
     signature = (a.shape, a.dtype, b.shape, b.dtype, acc_dtype, output_dtype)  # as the caller passed them
     if output_dtype is None:
         output_dtype = a.dtype
     acc_dtype, output_dtype = data_type(acc_dtype), data_type(output_dtype)
     if acc_dtype != torch.float32:
         raise ValueError('matmul_f8 accumulates in float32 only, got acc_dtype {}'.format(acc_dtype))
-    if output_dtype not in _OUT_TYPES:
-        raise ValueError('unsupported output dtype {}'.format(output_dtype))
+    if output_dtype not in _OUT_TYPES or (output_dtype in (f8e4m3, f8e5m2) and output_dtype != a.dtype):
+        raise ValueError('unsupported output dtype {} for operands of {}'.format(output_dtype, a.dtype))
     if is_scaled:
         return MatmulF8ScaledOperator(a, b, scale_a, scale_b, acc_dtype, output_dtype, bias).outputs[0]
     c = MatmulF8Operator(a, b, acc_dtype, output_dtype).outputs[0]

@@ -41,7 +41,8 @@ enum {
     HIDET_QMM_BF16 = 2,
     HIDET_QMM_I8 = 3,
     HIDET_QMM_I16 = 4,
-    HIDET_QMM_E4M3 = 5 /* OCP float8 e4m3fn: max 448, no infinities */
+    HIDET_QMM_E4M3 = 5, /* OCP float8 e4m3fn: max 448, no infinities */
+    HIDET_QMM_E5M2 = 6  /* OCP float8 e5m2: max 57344 */
 };
 
 /* ---- error state: same two symbols, same semantics as the reference runtime ------------------
@@ -169,6 +170,12 @@ void hidet_fp8_quantize_per_tensor(const void *x, void *codes, void *scale, int6
 void hidet_matmul_f8(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
                      int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
                      void *stream);
+/* The same task for float8_e5m2 operands (the reference accepts both operands e4m3 or both e5m2,
+ * python/hidet/graph/ops/matmul/matmul_f8.py:709-712): same arguments and meaning as hidet_matmul_f8 without the
+ * workspace; out_dtype float8_e5m2, float16, bfloat16 or float32 (conversion to e5m2 rounds to nearest even and
+ * saturates at +-57344). Served by the MFMA's bf8 format on a plainer kernel than the e4m3 one. */
+void hidet_matmul_f8_e5m2(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
+                          int out_dtype, const void *scale_a, const void *scale_b, void *stream);
 /* replaces MatmulF8ScaledTask (python/hidet/graph/ops/matmul/matmul_f8.py:357-454, 632-636): per K block of
  * 128, c += (sum_{k in block} a * b) * scale_a[kb, m] * scale_b[n / 128, kb]; scale_a float32 [k/128, m],
  * scale_b float32 [n/128, k/128]; a [m, k] and b [n, k] dense. */

@@ -343,6 +343,44 @@ def e4m3_encode(x: np.ndarray) -> np.ndarray:
     return (idx | sign).astype(np.uint8)
 
 
+# --------------------------------------------------------------------------------------
+# FP8 e5m2 (OCP): bias 15, max 57344 (0x7B), 0x7C infinity, 0x7D-0x7F NaN, subnormals to 2**-16. A code is
+# the upper byte of the float16 with the same value. Conversion from float32 rounds to nearest even and
+# saturates finite values AND infinities to +-57344, NaN -> 0x7F: the saturate-to-finite conversion of the
+# reference's float8_e5m2 type (include/hidet/runtime/cuda/float8_e5m2.h:6).
+# --------------------------------------------------------------------------------------
+
+def e5m2_decode(code: np.ndarray) -> np.ndarray:
+    c = np.asarray(code, dtype=np.uint8).astype(np.uint16)
+    return (c << np.uint16(8)).astype(np.uint16).view(np.float16).astype(np.float32)
+
+
+_E5M2_POS = None
+
+
+def _e5m2_pos_table() -> np.ndarray:
+    global _E5M2_POS
+    if _E5M2_POS is None:
+        _E5M2_POS = e5m2_decode(np.arange(0x7C, dtype=np.uint8)).astype(np.float64)  # 0 .. 57344, ascending
+    return _E5M2_POS
+
+
+def e5m2_encode(x: np.ndarray) -> np.ndarray:
+    """float32 -> e5m2 code by search in the table of the 124 non-negative finite values (ties to the even code)."""
+    x = np.asarray(x, dtype=np.float32)
+    tab = _e5m2_pos_table()
+    ax = np.minimum(np.abs(x.astype(np.float64)), 57344.0)
+    ax = np.where(np.isnan(ax), 0.0, ax)
+    hi = np.clip(np.searchsorted(tab, ax, side='left'), 0, len(tab) - 1)
+    lo = np.clip(hi - 1, 0, len(tab) - 1)
+    d_hi, d_lo = tab[hi] - ax, ax - tab[lo]
+    pick_lo = (d_lo < d_hi) | ((d_lo == d_hi) & ((lo & 1) == 0))
+    idx = np.where(pick_lo, lo, hi).astype(np.uint8)
+    idx = np.where(np.isnan(x), np.uint8(0x7F), idx)
+    sign = (np.signbit(x).astype(np.uint8) << 7).astype(np.uint8)
+    return (idx | sign).astype(np.uint8)
+
+
 def fp8_quantize_per_tensor(x: np.ndarray) -> Tuple[np.ndarray, np.float32]:
     """scale = amax / 448 (float32), code = e4m3(x / scale)  (benchmark-defined)."""
     x = np.asarray(x, dtype=np.float32)
@@ -355,16 +393,21 @@ def fp8_quantize_per_tensor(x: np.ndarray) -> Tuple[np.ndarray, np.float32]:
 def _cast_out(c32: np.ndarray, out_dtype: str) -> np.ndarray:
     if out_dtype == 'float8_e4m3':
         return e4m3_encode(c32)
+    if out_dtype == 'float8_e5m2':
+        return e5m2_encode(c32)
     return _round_to(c32, out_dtype)
 
 
-def matmul_f8(a_code: np.ndarray, b_code: np.ndarray, out_dtype: str = 'float8_e4m3', acc: str = 'f32') -> np.ndarray:
+def matmul_f8(a_code: np.ndarray, b_code: np.ndarray, out_dtype: Union[str, None] = None, acc: str = 'f32',
+              in_dtype: str = 'float8_e4m3') -> np.ndarray:
     """C[..., M, N] = cast(sum_k f32(A[..., M, k]) * f32(B[..., N, k])); A is [M, K] and B is
-    [N, K], both K-major (graph/ops/matmul/matmul_f8.py:132-149, 693-742).  The default output
-    dtype is the input fp8 type (:714-715)."""
+    [N, K], both K-major and both of `in_dtype`, float8_e4m3 or float8_e5m2 (graph/ops/matmul/matmul_f8.py:132-149,
+    693-742).  The default output dtype is the input fp8 type (:714-715)."""
     t = np.float64 if acc == 'f64' else np.float32
-    a = e4m3_decode(a_code).astype(t)
-    b = e4m3_decode(b_code).astype(t)
+    decode = e5m2_decode if in_dtype == 'float8_e5m2' else e4m3_decode
+    out_dtype = in_dtype if out_dtype is None else out_dtype
+    a = decode(a_code).astype(t)
+    b = decode(b_code).astype(t)
     c = np.matmul(a, np.swapaxes(b, -1, -2)).astype(np.float32)
     return _cast_out(c, out_dtype)
 

@@ -243,6 +243,58 @@ def test_per_tensor_exact_case(m, k, n):
                                                                  np.float32(sa), np.float32(sb), 'float32'))
 
 
+@pytest.mark.parametrize('a_shape, b_shape', [[[256, 128], [256, 128]], [[512, 256], [128, 256]], [[1, 256], [48, 256]],
+                                              [[16, 1024], [200, 1024]], [[100, 48], [36, 48]], [[300, 272], [260, 272]],
+                                              [[7, 100], [33, 100]], [[1000, 512], [520, 512]]])
+def test_matmul_f8_e5m2_reference_recipe(a_shape, b_shape):
+    # the reference accepts both operands float8_e5m2 as well (matmul_f8.py:709-712); same integer recipe
+    # (tests/operators_core/test_matmul.py:250-288). Up to 16 rows: the bandwidth-bound kernel; aligned shapes: the tile
+    # kernel on the MFMA's bf8 format; the rest: the element-wise kernel.
+    announce('matmul_f8 e5m2', a_shape, b_shape)
+    rng = np.random.default_rng(44)
+    ai, bi = rng.integers(-3, 3, a_shape), rng.integers(-3, 3, b_shape)
+    ta = dev(O.e5m2_encode(ai.astype(np.float32))).view(torch.float8_e5m2)
+    tb = dev(O.e5m2_encode(bi.astype(np.float32))).view(torch.float8_e5m2)
+    exact = (ai.astype(np.float64) @ bi.astype(np.float64).T).astype(np.int64)
+    got32 = F8.matmul_f8(ta, tb, output_dtype='float32')
+    assert np.array_equal(host(got32).astype(np.int64), exact)
+    got8 = F8.matmul_f8(ta, tb)
+    assert got8.dtype == torch.float8_e5m2
+    assert np.array_equal(got8.view(torch.uint8).cpu().numpy(), O.e5m2_encode(exact.astype(np.float32)))
+    gotb = F8.matmul_f8(ta, tb, output_dtype='bfloat16')
+    assert np.array_equal(host(gotb), O.to_bf16(exact.astype(np.float32)))
+    assert np.array_equal(host(got32), O.matmul_f8(host(ta.view(torch.uint8)), host(tb.view(torch.uint8)), 'float32',
+                                                   in_dtype='float8_e5m2'))
+
+
+def test_e5m2_output_conversion_every_boundary():
+    # float32 -> e5m2 in the epilogue: a 1 x 1 x K product that lands on every midpoint between neighbouring codes
+    # and just beside it, plus saturation; a = [x, 0, ...] in e5m2 cannot carry these values, so the values are built
+    # as sums of two exactly representable operands: x = hi + lo with b = [1, 1, 0, ...]
+    announce('e5m2 output rounding')
+    tab = O.e5m2_decode(np.arange(0x7C, dtype=np.uint8)).astype(np.float64)
+    cases = []
+    for i in range(0x10, 0x7B):  # normal range: midpoint = tab[i] + half a step, half a step is itself a code value
+        half = (tab[i + 1] - tab[i]) / 2
+        if O.e5m2_decode(O.e5m2_encode(np.array([half], dtype=np.float32)))[0] == half:
+            cases.append((tab[i], half))
+    hi = np.array([c[0] for c in cases], dtype=np.float32)
+    lo = np.array([c[1] for c in cases], dtype=np.float32)
+    a = np.zeros((len(cases), 16), dtype=np.float32)
+    a[:, 0], a[:, 1] = hi, lo
+    b = np.zeros((4, 16), dtype=np.float32)
+    b[0, :2] = 1.0
+    b[1, 0] = 1.0
+    ta = dev(O.e5m2_encode(a)).view(torch.float8_e5m2)
+    tb = dev(O.e5m2_encode(b)).view(torch.float8_e5m2)
+    got = F8.matmul_f8(ta, tb).view(torch.uint8).cpu().numpy()
+    want = O.e5m2_encode((hi.astype(np.float64) + lo.astype(np.float64)).astype(np.float32))
+    assert np.array_equal(got[:, 0], want) and np.array_equal(got[:, 1], O.e5m2_encode(hi))
+    big = dev(O.e5m2_encode(np.full((2, 16), 57344.0, dtype=np.float32))).view(torch.float8_e5m2)
+    ones = dev(O.e5m2_encode(np.ones((4, 16), dtype=np.float32))).view(torch.float8_e5m2)
+    assert set(F8.matmul_f8(big, ones).view(torch.uint8).cpu().numpy().ravel().tolist()) == {0x7B}  # saturates, no infinity
+
+
 def test_expanded_and_transposed_operands():
     # operands whose rows cannot be addressed with a stride >= K (one row expanded to M rows, a transposed view) are
     # copied by the operator before they reach the kernel
@@ -290,6 +342,8 @@ def test_argument_errors():
     with pytest.raises(ValueError, match=r'\[\.\.\.,M,K\] and \[\.\.\.,N,K\]'):
         F8.matmul_f8(a, torch.zeros(4, 32, device='cuda').to(torch.float8_e4m3fn))
     with pytest.raises(NotImplementedError):
-        F8.matmul_f8(a.to(torch.float8_e5m2), a.to(torch.float8_e5m2))
+        F8.matmul_f8_scaled(a.to(torch.float8_e5m2), a.to(torch.float8_e5m2), torch.ones(1, 4, device='cuda'), torch.ones(1, 1, device='cuda'))
+    with pytest.raises(ValueError, match='unsupported output dtype'):
+        F8.matmul_f8(a, a, output_dtype='float8_e5m2')
     with pytest.raises(ValueError, match='bias is not supported'):
         F8.matmul_f8_scaled(a, a, torch.ones(1, 4, device='cuda'), torch.ones(1, 1, device='cuda'), bias=torch.ones(4, device='cuda'))

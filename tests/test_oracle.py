@@ -446,6 +446,46 @@ def test_matmul_f8_scaled_reference_recipe():
     assert np.array_equal(got.astype(np.int64), a2 @ b2.T)
 
 
+def test_e5m2_codec_against_torch_and_float16():
+    # decode: every code against torch.float8_e5m2 and against "upper byte of the float16 of the same value"
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+    got = O.e5m2_decode(codes)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+    assert got[0x7B] == 57344.0 and np.isinf(got[0x7C]) and got[0x01] == 2.0 ** -16 and got[0x04] == 2.0 ** -14
+    # encode: round to nearest even against torch inside the finite range (torch overflows to infinity beyond it, the
+    # reference's type saturates: checked separately), every midpoint between neighbouring codes included
+    tab = got[:0x7C].astype(np.float64)
+    mids = (tab[:-1] + tab[1:]) / 2
+    rng = np.random.default_rng(2)
+    xs = np.concatenate([tab, mids, np.nextafter(mids.astype(np.float32), np.float32(0)).astype(np.float64),
+                         np.nextafter(mids.astype(np.float32), np.float32(1e9)).astype(np.float64),
+                         rng.standard_normal(4000) * 100, rng.standard_normal(4000) * 1e-4]).astype(np.float32)
+    xs = np.concatenate([xs, -xs])
+    xs = xs[np.abs(xs) <= 57344]
+    want = torch.from_numpy(xs).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    assert np.array_equal(O.e5m2_encode(xs), want)
+    # saturation and NaN of the reference's conversion
+    sat = O.e5m2_encode(np.array([57344.0, 60000.0, 65504.0, 1e9, np.inf, -1e9, -np.inf, 61439.9], dtype=np.float32))
+    assert sat.tolist() == [0x7B, 0x7B, 0x7B, 0x7B, 0x7B, 0xFB, 0xFB, 0x7B]
+    assert (O.e5m2_encode(np.array([np.nan], dtype=np.float32))[0] & 0x7F) == 0x7F
+    assert O.e5m2_encode(np.array([2.0 ** -17, 2.0 ** -17 * 1.0001, 3 * 2.0 ** -17], dtype=np.float32)).tolist() == [0, 1, 2]
+
+
+def test_matmul_f8_e5m2_reference_recipe():
+    # tests/operators_core/test_matmul.py:250-288 with float8_e5m2 operands: small integers, exact result
+    rng = np.random.default_rng(43)
+    ai, bi = rng.integers(-3, 3, (20, 96)), rng.integers(-3, 3, (12, 96))
+    ac, bc = O.e5m2_encode(ai.astype(np.float32)), O.e5m2_encode(bi.astype(np.float32))
+    assert np.array_equal(O.e5m2_decode(ac), ai) and np.array_equal(O.e5m2_decode(bc), bi)
+    exact = ai.astype(np.int64) @ bi.astype(np.int64).T
+    assert np.array_equal(O.matmul_f8(ac, bc, out_dtype='float32', in_dtype='float8_e5m2').astype(np.int64), exact)
+    got8 = O.matmul_f8(ac, bc, in_dtype='float8_e5m2')  # default output: the input type
+    assert np.array_equal(got8, O.e5m2_encode(exact.astype(np.float32)))
+    # the same codes read as e4m3 are different numbers: the decode table matters
+    assert not np.array_equal(O.matmul_f8(ac, bc, out_dtype='float32'), exact)
+
+
 def test_fp8_per_tensor_quantize_and_matmul():
     a32, b32 = O.make_inputs(0, 32, 256, 48)
     b32 = b32.T.copy()  # [N, K]
