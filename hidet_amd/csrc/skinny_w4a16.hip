@@ -16,14 +16,20 @@
 namespace qmm {
 namespace {
 
-constexpr int kSkinnyWaves = 4;  // waves per workgroup; they split the workgroup's K slice
+constexpr int kSkinnyWaves = 8;   // waves per workgroup; they split the workgroup's K slice
+constexpr int kNonTemporal = 2;   // cache policy bits of a buffer load: sc0 = 1, nt = 2, sc1 = 16
+constexpr int kDepth = 2;          // 32-row steps fetched together
 
-template <int DT, int DEPTH, bool ALIGNED_A, bool FULL = false>
-__global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,
-                                                           const uint8_t *__restrict__ w,
-                                                           const uint16_t *__restrict__ scales, uint16_t *__restrict__ c,
-                                                           int m, int k, int n, int group, int rows_per_block, int splits,
-                                                           int tiles, float *__restrict__ mailbox) {
+// Same launch shape and load discipline as the int8 kernel: 8-wave workgroups in one round over the chip, one 32-row
+// step (8 loads of 8 bytes per lane, non-temporal) in flight per wave, no condition around a load - rows past the wave's
+// range lie outside the buffer and read as zero bytes, which are code 0 - and the split-K exchange of skinny_finish.
+template <int DT, bool ALIGNED_A>
+__global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,
+                                                                        const uint8_t *__restrict__ w,
+                                                                        const uint16_t *__restrict__ scales,
+                                                                        uint16_t *__restrict__ c, int m, int k, int n, int group,
+                                                                        int rows_per_block, int splits, int tiles,
+                                                                        float *__restrict__ mailbox) {
     using T = W4Traits<DT>;
     extern __shared__ float red[];
 
@@ -31,15 +37,17 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
     if (!skinny_tile_of_block(splits, tiles, &tile, &split)) return;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, cl = lane & 15;
-    const int col0 = tile * kSkinnyTileN + cl * 16;
-    const bool col_ok = col0 < n;
-    const int64_t row_bytes = n >> 1;
+    const int tile_col = tile * kSkinnyTileN;
+    const bool col_ok = tile_col + cl * 16 < n;
+    const int row_bytes = n >> 1;
 
     const int rows_per_wave = rows_per_block / kSkinnyWaves;
     const int k_begin = split * rows_per_block + wave * rows_per_wave;
     const int k_end = min(k, k_begin + rows_per_wave);
+    const int nsteps = k_end > k_begin ? (k_end - k_begin + 31) >> 5 : 0;
 
     float4_t acc[16], total[16];
 #pragma unroll
@@ -51,98 +59,98 @@ __global__ __launch_bounds__(256, 2) void skinny_w4a16_kernel(const uint16_t *__
     const uint32_t one2 = uint32_t(T::kOne) | (uint32_t(T::kOne) << 16);
     const uint4 ones = uint4{one2, one2, one2, one2};
 
-    // FULL: every column exists, every wave's K range is a whole number of iterations and the activations allow 16-byte
-    // loads, so the loop has no per-lane conditions; lanes of rows >= M read the last row and their results are dropped
-    const uint8_t *wp = w + (col0 >> 1);
-    const uint16_t *ap = a + int64_t(FULL ? min(cl, m - 1) : cl) * lda;
-    uint4 sc_raw[2] = {uint4{0u, 0u, 0u, 0u}, uint4{0u, 0u, 0u, 0u}};  // 16 scales of the current group
+    // weights: the wave's rows at the tile's first byte column; a lane whose 16 columns lie past N reads the tile's
+    // first columns and its results are never stored
+    const int64_t w_bytes = int64_t(k_end - k_begin) * row_bytes - (tile_col >> 1);
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t *>(w + int64_t(k_begin) * row_bytes + (tile_col >> 1)), 0, int(w_bytes < 0 ? 0 : w_bytes), 0x00020000);
+    uint32_t w_off = uint32_t(8 * g) * uint32_t(row_bytes) + (col_ok ? cl * 8 : 0);
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(a), 0, ALIGNED_A ? int((int64_t(m - 1) * lda + k) * 2) : 0, 0x00020000);
+    const uint16_t *ap = a + int64_t(cl) * lda;
+    const int a_row_off = int(int64_t(cl) * lda * 2);
+    // scales of this lane's 16 columns: 32 bytes per group
+    const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(scales), 0, int(int64_t(k / group) * n * 2), 0x00020000);
+    const int s_col_off = (tile_col + (col_ok ? cl * 16 : 0)) * 2;
+    uint4v_t sc_raw[2] = {uint4v_t{0u, 0u, 0u, 0u}, uint4v_t{0u, 0u, 0u, 0u}};
 
-    for (int kk = k_begin; kk < k_end; kk += 32 * DEPTH) {
-        uint2 raw[DEPTH][8];
-        uint4 xa[DEPTH];
+    // kDepth 32-row steps are fetched together: a step is only 4 KiB per wave here (8 bytes per lane and row). Measured at
+    // 4096 x 11008, one row: 1 / 2 / 4 steps 9.5 / 9.3 / 9.9 us; without any of the arithmetic below 8.3 - 8.6 us: the
+    // kernel's time is launch ramp, memory latency and the exchange, not the 23 MB it reads.
+    for (int step0 = 0; step0 < nsteps; step0 += kDepth) {
+        uint2 raw[kDepth][8];
+        uint4 xa[kDepth];
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d)
+        for (int d = 0; d < kDepth; ++d) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int row = kk + 32 * d + 8 * g + j;
-                if (FULL) {
-                    raw[d][j] = *reinterpret_cast<const uint2 *>(wp + int64_t(row) * row_bytes);
-                    continue;
-                }
-                raw[d][j] = uint2{0x88888888u, 0x88888888u};  // nibble 8 ^ 8 == code 0
-                if (col_ok && row < k_end) raw[d][j] = *reinterpret_cast<const uint2 *>(wp + int64_t(row) * row_bytes);
+            for (int r = 0; r < 8; ++r) {
+                const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_off + uint32_t(r) * uint32_t(row_bytes), 0, kNonTemporal);
+                raw[d][r] = uint2{v[0], v[1]};
             }
+            w_off += 32u * uint32_t(row_bytes);
+            asm volatile("" : "+v"(w_off));
+            const int kx = k_begin + 32 * (step0 + d) + 8 * g;
+            if (ALIGNED_A) {
+                const int off = (cl < m && kx < k_end) ? a_row_off + kx * 2 : 0x7FFFFFF0;
+                xa[d] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0));
+            } else {
+                uint16_t tmp[8];
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const int kx = kk + 32 * d + 8 * g;
-            if (FULL) {
-                xa[d] = *reinterpret_cast<const uint4 *>(ap + kx);
-                continue;
-            }
-            xa[d] = uint4{0u, 0u, 0u, 0u};
-            if (cl < m) {
-                if (ALIGNED_A) {
-                    if (kx < k_end) xa[d] = *reinterpret_cast<const uint4 *>(ap + kx);
-                } else {
-                    uint16_t tmp[8];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) tmp[j] = (kx + j < k_end) ? ap[kx + j] : uint16_t(0);
-                    xa[d] = uint4{uint32_t(tmp[0]) | (uint32_t(tmp[1]) << 16), uint32_t(tmp[2]) | (uint32_t(tmp[3]) << 16),
-                                  uint32_t(tmp[4]) | (uint32_t(tmp[5]) << 16), uint32_t(tmp[6]) | (uint32_t(tmp[7]) << 16)};
-                }
+                for (int j = 0; j < 8; ++j) tmp[j] = (cl < m && kx + j < k_end) ? ap[kx + j] : uint16_t(0);
+                xa[d] = uint4{uint32_t(tmp[0]) | (uint32_t(tmp[1]) << 16), uint32_t(tmp[2]) | (uint32_t(tmp[3]) << 16),
+                              uint32_t(tmp[4]) | (uint32_t(tmp[5]) << 16), uint32_t(tmp[6]) | (uint32_t(tmp[7]) << 16)};
             }
         }
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const int ks = kk + 32 * d;
-            if (FULL || ks < k_end) {  // uniform across the wave
-                if (ks % group == 0 || ks == k_begin) {
-                    if (FULL || col_ok) {
-                        const uint16_t *sp = scales + int64_t(ks / group) * n + col0;
-                        sc_raw[0] = *reinterpret_cast<const uint4 *>(sp);
-                        sc_raw[1] = *reinterpret_cast<const uint4 *>(sp + 8);
+        for (int d = 0; d < kDepth; ++d) {
+            const int step = step0 + d;
+            if (step >= nsteps) break;  // uniform across the wave
+            const int ks = k_begin + 32 * step;
+            if (ks % group == 0 || step == 0) {  // a new group starts
+                const int soff = (ks / group) * n * 2 + s_col_off;
+                sc_raw[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, soff, 0, 0);
+                sc_raw[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, soff + 16, 0, 0);
+            }
+            // byte b of dword h of rows 2p and 2p+1 goes to bits 0-7 and 16-23 of one register (v_perm_b32); its low
+            // nibbles are column 8h + 2b of both rows, its high nibbles column 8h + 2b + 1: mask-and-xor (one
+            // three-input bit operation) gives the two 16-bit floats bias + q, for the odd column after a shift
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int byte = 0; byte < 4; ++byte) {
+                    constexpr uint32_t kZero = 0x0c;
+                    const uint32_t sel = (kZero << 24) | (uint32_t(4 + byte) << 16) | (kZero << 8) | uint32_t(byte);
+                    uint4 be, bo;
+                    uint32_t *bep = reinterpret_cast<uint32_t *>(&be), *bop = reinterpret_cast<uint32_t *>(&bo);
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const uint32_t lo = h ? raw[d][2 * p].y : raw[d][2 * p].x;
+                        const uint32_t hi = h ? raw[d][2 * p + 1].y : raw[d][2 * p + 1].x;
+                        const uint32_t x = __builtin_amdgcn_perm(hi, lo, sel);
+                        bep[p] = (x & 0x000F000Fu) ^ T::kMagic;
+                        bop[p] = ((x >> 4) & 0x000F000Fu) ^ T::kMagic;
+                    }
+                    const int t = 8 * h + 2 * byte;
+                    acc[t] = T::mfma(xa[d], be, acc[t]);
+                    acc[t + 1] = T::mfma(xa[d], bo, acc[t + 1]);
+                }
+            }
+            xsum = T::mfma(xa[d], ones, xsum);
+            if ((ks + 32) % group == 0 || step == nsteps - 1) {  // group complete (or the wave's range ends): fold it in
+                const uint16_t *sv = reinterpret_cast<const uint16_t *>(sc_raw);
+#pragma unroll
+                for (int t = 0; t < 16; ++t) {
+                    const float s = T::to_f32(sv[t]);
+                    const float sb = -T::kBias * s;  // exact: a power of two plus a small multiple times a 16-bit float
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        total[t][v] = fmaf(acc[t][v], s, total[t][v]);
+                        total[t][v] = fmaf(xsum[v], sb, total[t][v]);
+                        acc[t][v] = 0.f;
                     }
                 }
-                // byte b of dword h of rows 2p and 2p+1 goes to bits 0-7 and 16-23 of one register (v_perm_b32); its low
-                // nibbles are column 8h + 2b of both rows, its high nibbles column 8h + 2b + 1: mask-and-xor (one
-                // three-input bit operation) gives the two 16-bit floats bias + q, for the odd column after a shift
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-#pragma unroll
-                    for (int byte = 0; byte < 4; ++byte) {
-                        constexpr uint32_t kZero = 0x0c;
-                        const uint32_t sel = (kZero << 24) | (uint32_t(4 + byte) << 16) | (kZero << 8) | uint32_t(byte);
-                        uint4 be, bo;
-                        uint32_t *bep = reinterpret_cast<uint32_t *>(&be), *bop = reinterpret_cast<uint32_t *>(&bo);
-#pragma unroll
-                        for (int p = 0; p < 4; ++p) {
-                            const uint32_t lo = h ? raw[d][2 * p].y : raw[d][2 * p].x;
-                            const uint32_t hi = h ? raw[d][2 * p + 1].y : raw[d][2 * p + 1].x;
-                            const uint32_t x = __builtin_amdgcn_perm(hi, lo, sel);
-                            bep[p] = (x & 0x000F000Fu) ^ T::kMagic;
-                            bop[p] = ((x >> 4) & 0x000F000Fu) ^ T::kMagic;
-                        }
-                        const int t = 8 * h + 2 * byte;
-                        acc[t] = T::mfma(xa[d], be, acc[t]);
-                        acc[t + 1] = T::mfma(xa[d], bo, acc[t + 1]);
-                    }
-                }
-                xsum = T::mfma(xa[d], ones, xsum);
-                if ((ks + 32) % group == 0 || ks + 32 >= k_end) {  // group complete (or slice ends): fold it in
-                    const uint16_t *sv = reinterpret_cast<const uint16_t *>(sc_raw);
-#pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        const float s = T::to_f32(sv[t]);
-                        const float sb = -T::kBias * s;  // exact: a power of two plus a small multiple times a 16-bit float
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            total[t][v] = fmaf(acc[t][v], s, total[t][v]);
-                            total[t][v] = fmaf(xsum[v], sb, total[t][v]);
-                            acc[t][v] = 0.f;
-                        }
-                    }
-                    xsum = float4_t{0.f, 0.f, 0.f, 0.f};
-                }
+                xsum = float4_t{0.f, 0.f, 0.f, 0.f};
             }
         }
     }
@@ -197,29 +205,34 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
         return;
     }
     int rpb, splits, tiles;
-    skinny_plan(k, n, 512, parallel_k_parts, 128, &rpb, &splits, &tiles);
+    skinny_plan_one_round(k, n, kSkinnyWaves, parallel_k_parts, &rpb, &splits, &tiles);
     const Workspace ws = split_workspace(workspace, workspace_bytes);
-    skinny_fit_mailbox(k, 128, tiles, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, &rpb, &splits);
-    const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16);
+    skinny_fit_mailbox(k, 32 * kSkinnyWaves, tiles, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, &rpb, &splits);
+    // a wave's K range and the scale table are addressed with 31-bit offsets
+    if ((int64_t(rpb) / kSkinnyWaves + 64) * (n / 2) >= (int64_t(1) << 31) - (1 << 20) || (k / group) * n * 2 >= (int64_t(1) << 31) - (1 << 20)) {
+        if (dtype == HIDET_QMM_F16)
+            launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
+        else
+            launch(naive_w4a16_kernel<HIDET_QMM_BF16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
+        return;
+    }
+    // 16-byte activation loads through a buffer descriptor: aligned rows, offsets below 2^31
+    const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16) && (15 * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
     const int grid = int(cdiv(tiles, 8) * 8 * splits);
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
         const size_t shmem = skinny_lds_bytes(mt, kSkinnyWaves);
         auto go = [&](auto kern) {
             if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16, kSkinnyWaves)));  // the most any m needs
-            launch(kern, dim3(grid), dim3(256), shmem, stream, ap0 + m0 * lda, lda, wp, sp, cp0 + m0 * n, mt, int(k), int(n),
-                   group, rpb, splits, tiles, ws.mailbox);
+            launch(kern, dim3(grid), dim3(64 * kSkinnyWaves), shmem, stream, ap0 + m0 * lda, lda, wp, sp, cp0 + m0 * n, mt, int(k),
+                   int(n), group, rpb, splits, tiles, ws.mailbox);
         };
-        const bool full = aligned_a && n % kSkinnyTileN == 0 && k % rpb == 0 && rpb % (kSkinnyWaves * 64) == 0;
-        if (full) {
-            if (dtype == HIDET_QMM_F16) go(skinny_w4a16_kernel<HIDET_QMM_F16, 2, true, true>);
-            else go(skinny_w4a16_kernel<HIDET_QMM_BF16, 2, true, true>);
-        } else if (dtype == HIDET_QMM_F16) {
-            if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, 2, true>);
-            else go(skinny_w4a16_kernel<HIDET_QMM_F16, 2, false>);
+        if (dtype == HIDET_QMM_F16) {
+            if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, true>);
+            else go(skinny_w4a16_kernel<HIDET_QMM_F16, false>);
         } else {
-            if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_BF16, 2, true>);
-            else go(skinny_w4a16_kernel<HIDET_QMM_BF16, 2, false>);
+            if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_BF16, true>);
+            else go(skinny_w4a16_kernel<HIDET_QMM_BF16, false>);
         }
     }
 }
