@@ -105,6 +105,9 @@ def main():
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--pmc-calibration', action='store_true',
                     help='short run for `rocprofv3 --pmc`: a few 64 MiB device copies of known traffic, then one pass over the GEMV ring')
+    ap.add_argument('--decode-counters', action='store_true',
+                    help='short run for `rocprofv3 --pmc`: the decode kernels of the smaller configurations only (W4A16 M = 1 and 16 '
+                         'at 4096 x 11008, W8A16 M = 16 at 4096 x 4096, the headline GEMV for comparison), over distinct weight buffers')
     ap.add_argument('--skip-two-chains', action='store_true',
                     help='leave out the two-stream graph: under a kernel trace its overlapping launches would blur the GEMV kernel\'s average duration')
     ap.add_argument('--data-dependence', action='store_true',
@@ -136,6 +139,32 @@ def main():
 
     def launch(i, st):
         ffi.call('hidet_symmetric_quant_matmul_f16_i8', a, ws[i], ss[i], outs[i], 1, K, N, K, 0, work, work.numel(), st)
+
+    if args.decode_counters:
+        g2 = torch.Generator(device=device)
+        g2.manual_seed(7)
+        w4 = [torch.randint(0, 256, (K, N // 2), device=device, dtype=torch.uint8) for _ in range(16)]
+        s4 = (torch.rand((K // 128, N), generator=g2, device=device) * 0.01 + 0.001).to(torch.bfloat16)
+        w16 = [torch.randint(-127, 128, (4096, 4096), device=device, dtype=torch.int8) for _ in range(16)]
+        a16 = torch.randn((16, 4096), generator=g2, device=device, dtype=torch.float32).to(torch.float16)
+        c16 = torch.empty((16, 4096), dtype=torch.float16, device=device)
+        s16 = ss[0][:4096].contiguous()
+        with torch.cuda.stream(stream):
+            for m4 in (1, 16):
+                a4 = torch.randn((m4, K), generator=g2, device=device, dtype=torch.float32).to(torch.bfloat16)
+                c4 = torch.empty((m4, N), dtype=torch.bfloat16, device=device)
+                for rep in range(2):
+                    for i in range(16):
+                        ffi.call('hidet_symmetric_quant_matmul_w4a16', a4, w4[i], s4, c4, m4, K, N, K, 128, 2, 0, work, work.numel(), sptr)
+            for rep in range(2):
+                for i in range(16):
+                    ffi.call('hidet_symmetric_quant_matmul_f16_i8', a16, w16[i], s16, c16, 16, 4096, 4096, 4096, 0, work, work.numel(), sptr)
+            for rep in range(2):
+                for i in range(RING):
+                    launch(i, sptr)
+        stream.synchronize()
+        print(json.dumps({'decode_counters': {'order': ['w4a16 m=1 x32', 'w4a16 m=16 x32', 'w8a16 m=16 4096x4096 x32', 'w8a16 gemv x32']}}))
+        return
 
     if args.pmc_calibration:
         src = torch.empty(64 << 20, dtype=torch.uint8, device=device).random_(0, 255)
@@ -412,19 +441,19 @@ def main():
     others['w8a16_m32_k4096_n11008'] = hbm_entry(us, K * N + 2 * N + 2 * 32 * (K + N))
     del wq, cq
     # group-wise W4A16 (bf16, group 128), M in {1, 16, 512}
-    w4 = [torch.randint(0, 256, (K, N // 2), device=device, dtype=torch.uint8) for _ in range(16)]
+    w4 = [torch.randint(0, 256, (K, N // 2), device=device, dtype=torch.uint8) for _ in range(24)]  # 24 x 22.5 MB = 541 MB > 2 x the LLC
     s4 = (torch.rand((K // 128, N), generator=g, device=device) * 0.01 + 0.001).to(torch.bfloat16)
     for m4 in (1, 16, 512):
         a4 = torch.randn((m4, K), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
         c4 = torch.empty((m4, N), dtype=torch.bfloat16, device=device)
-        us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16', a4, w4[r % 16], s4, c4, m4, K, N, K, 128, 2, 0,
-                                          work, work.numel(), sptr), 40, 16)
+        us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16', a4, w4[r % 24], s4, c4, m4, K, N, K, 128, 2, 0,
+                                          work, work.numel(), sptr), 48, 24)
         nbytes = K * N // 2 + 2 * (K // 128) * N + 2 * m4 * K + 2 * m4 * N
         others['w4a16_m{}_k4096_n11008'.format(m4)] = (hbm_entry(us, nbytes) if m4 <= 16 else
                                                       mfma_entry(us, 2.0 * m4 * K * N, MFMA_F16_PEAK_TFLOPS))
         if m4 <= 16:  # the same bytes read as the [N, K/2] decode layout (another data layout: never the headline)
-            us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16_nk', a4, w4[r % 16].view(N, K // 2), s4, c4, m4, K, N,
-                                              K, K // 2, 128, 2, sptr), 40, 16)
+            us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16_nk', a4, w4[r % 24].view(N, K // 2), s4, c4, m4, K, N,
+                                              K, K // 2, 128, 2, sptr), 48, 24)
             others['w4a16_m{}_k4096_n11008_decode_layout'.format(m4)] = hbm_entry(us, nbytes)
     del w4
     # FP8 decode variant: M = 1 against the same b
