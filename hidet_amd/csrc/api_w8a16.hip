@@ -2,19 +2,19 @@
 #include "common.h"
 
 namespace qmm {
-void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace,
-                         hipStream_t stream);
+void skinny_w8a16_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                         int64_t n, int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes,
+                         bool strict_workspace, hipStream_t stream);
 bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda);
-void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                       int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+void gemm_w8a16_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                       int64_t n, int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 bool skinny_w8a16_nk_supported(const void *w, int64_t k, int64_t ldw);
-void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                            int64_t lda, int64_t ldw, hipStream_t stream);
+void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                            int64_t n, int64_t lda, int64_t ldw, hipStream_t stream);
 bool gemm_w8a16_nk_supported(const void *a, const void *w, const void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
                              int64_t ldw);
-void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                          int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                          int64_t n, int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream);
 }
 
 using namespace qmm;
@@ -23,15 +23,16 @@ namespace {
 
 // Checks and kernel choice shared by the two row-major entry points. `strict_workspace`: a bandwidth-bound launch whose
 // K split does not fit the scratch memory is an error instead of a launch with fewer K slices.
-void w8a16_dispatch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
-                    int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace, hipStream_t stream) {
+void w8a16_dispatch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k, int64_t n,
+                    int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace,
+                    hipStream_t stream) {
     QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
     QMM_CHECK(lda >= k, "row stride of a (" << lda << ") is smaller than K (" << k << ")");
     QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
     QMM_CHECK(parallel_k_parts >= 0, "parallel_k_parts must be >= 0");
     if (m == 0 || n == 0) return;
     QMM_CHECK(a && w && scale && c, "null tensor pointer");
-    QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
+    QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2) && aligned(bias, 2), "float16 tensors must be 2-byte aligned");
     // Up to 16 rows one pass of the bandwidth-bound kernel serves; beyond that every 16 rows would cost another pass
     // over the weights, and the MFMA GEMM with its K split and its empty row blocks left out takes over (K=4096, N=11008,
     // weights from HBM: 17 us at M=17..32, 20 us at M=64, 29 us at M=128). From 9 rows on the GEMM is already ahead when
@@ -39,10 +40,32 @@ void w8a16_dispatch(const void *a, const void *w, const void *scale, void *c, in
     // against 13.4 us), unless the caller asked for a specific K split of the bandwidth-bound kernel.
     const bool wide = cdiv(n, 256) >= 32;
     if ((m > 16 || (m > 8 && wide && parallel_k_parts == 0)) && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
-        gemm_w8a16_launch(a, w, scale, c, m, k, n, lda, workspace, workspace_bytes, stream);
+        gemm_w8a16_launch(a, w, scale, bias, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
-        skinny_w8a16_launch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, strict_workspace,
+        skinny_w8a16_launch(a, w, scale, bias, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, strict_workspace,
                             stream);
+}
+
+// Checks and kernel choice shared by the two entry points for K-contiguous weights.
+void w8a16_nk_dispatch(const void *a, const void *w_nk, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                       int64_t n, int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
+    QMM_CHECK(lda >= k && ldw >= k, "row strides (" << lda << ", " << ldw << ") must be at least K (" << k << ")");
+    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
+    QMM_CHECK(workspace_bytes >= 0 && (workspace == nullptr || aligned(workspace, 16)),
+              "the workspace must be 16-byte aligned (or NULL: no tile is computed in K ranges)");
+    if (m == 0 || n == 0) return;
+    QMM_CHECK(a && w_nk && scale && c, "null tensor pointer");
+    QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2) && aligned(bias, 2), "float16 tensors must be 2-byte aligned");
+    QMM_CHECK(skinny_w8a16_nk_supported(w_nk, k, ldw),
+              "K-contiguous weights need K and the row stride to be multiples of 16 and a 16-byte aligned pointer, got K=" << k
+                                                                                                                         << " ldw=" << ldw);
+    // more than one pass of 16 rows: the MFMA GEMM reading the same layout, where its conditions hold
+    if (m > 16 && gemm_w8a16_nk_supported(a, w_nk, c, m, k, n, lda, ldw))
+        gemm_w8a16_nk_launch(a, w_nk, scale, bias, c, m, k, n, lda, ldw, workspace ? workspace : nullptr,
+                             workspace ? workspace_bytes : 0, stream);
+    else
+        skinny_w8a16_nk_launch(a, w_nk, scale, bias, c, m, k, n, lda, ldw, stream);
 }
 
 // Scratch memory of hidet_symmetric_quant_matmul_f16_i8_static, used exactly like a caller's workspace of that size
@@ -78,7 +101,7 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
                                                    int64_t k, int64_t n, int64_t lda, int parallel_k_parts,
                                                    void *workspace, int64_t workspace_bytes, void *stream_) {
     QMM_ENTRY_BEGIN
-    w8a16_dispatch(a, w, scale, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, false,
+    w8a16_dispatch(a, w, scale, nullptr, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, false,
                    static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }
@@ -90,7 +113,17 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8_static(const void *a, const v
                                                           void *stream_) {
     QMM_ENTRY_BEGIN
     void *ptr = static_scratch_of_current_device();
-    w8a16_dispatch(a, w, scale, c, m, k, n, lda, parallel_k_parts, ptr, kStaticScratchBytes, true,
+    w8a16_dispatch(a, w, scale, nullptr, c, m, k, n, lda, parallel_k_parts, ptr, kStaticScratchBytes, true,
+                   static_cast<hipStream_t>(stream_));
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_symmetric_quant_matmul_f16_i8_bias(const void *a, const void *w, const void *scale, const void *bias,
+                                                        void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
+                                                        int parallel_k_parts, void *workspace, int64_t workspace_bytes,
+                                                        void *stream_) {
+    QMM_ENTRY_BEGIN
+    w8a16_dispatch(a, w, scale, bias, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, false,
                    static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }
@@ -99,23 +132,14 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8_nk(const void *a, const void 
                                                       int64_t k, int64_t n, int64_t lda, int64_t ldw, void *workspace,
                                                       int64_t workspace_bytes, void *stream_) {
     QMM_ENTRY_BEGIN
-    QMM_CHECK(m >= 0 && k >= 0 && n >= 0, "negative extent: m=" << m << " k=" << k << " n=" << n);
-    QMM_CHECK(lda >= k && ldw >= k, "row strides (" << lda << ", " << ldw << ") must be at least K (" << k << ")");
-    QMM_CHECK(k < (int64_t(1) << 31) && n < (int64_t(1) << 31) && m < (int64_t(1) << 31), "extent exceeds 2^31");
-    QMM_CHECK(workspace_bytes >= 0 && (workspace == nullptr || aligned(workspace, 16)),
-              "the workspace must be 16-byte aligned (or NULL: no tile is computed in K ranges)");
-    if (m == 0 || n == 0) return;
-    QMM_CHECK(a && w_nk && scale && c, "null tensor pointer");
-    QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2), "float16 tensors must be 2-byte aligned");
-    QMM_CHECK(skinny_w8a16_nk_supported(w_nk, k, ldw),
-              "K-contiguous weights need K and the row stride to be multiples of 16 and a 16-byte aligned pointer, got K=" << k
-                                                                                                                         << " ldw=" << ldw);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
-    // more than one pass of 16 rows: the MFMA GEMM reading the same layout, where its conditions hold
-    if (m > 16 && gemm_w8a16_nk_supported(a, w_nk, c, m, k, n, lda, ldw))
-        gemm_w8a16_nk_launch(a, w_nk, scale, c, m, k, n, lda, ldw, workspace ? workspace : nullptr,
-                             workspace ? workspace_bytes : 0, stream);
-    else
-        skinny_w8a16_nk_launch(a, w_nk, scale, c, m, k, n, lda, ldw, stream);
+    w8a16_nk_dispatch(a, w_nk, scale, nullptr, c, m, k, n, lda, ldw, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_symmetric_quant_matmul_f16_i8_nk_bias(const void *a, const void *w_nk, const void *scale, const void *bias,
+                                                           void *c, int64_t m, int64_t k, int64_t n, int64_t lda, int64_t ldw,
+                                                           void *workspace, int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    w8a16_nk_dispatch(a, w_nk, scale, bias, c, m, k, n, lda, ldw, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

@@ -47,6 +47,7 @@ template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA, bool W_NK = false>
 __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(const _Float16 *__restrict__ a, int64_t lda,
                                                                                  const int8_t *__restrict__ w, int64_t ldw,
                                                                                  const _Float16 *__restrict__ scale,
+                                                                                 const _Float16 *__restrict__ bias,
                                                                                  _Float16 *__restrict__ c, int m, int k, int n,
                                                                                  int tiles_m, int tiles_n, int xm, int xn,
                                                                                  int concurrent, int tail_parts, int tail_stride,
@@ -283,9 +284,12 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
 
     // acc[rb][t][v] = c[m0 + (wm*RB + rb)*16 + 4*kg + v][col + t]
     if (!col_ok) return;
-    float sc[4];
+    float sc[4], bs[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) sc[t] = float(scale[col + t]);
+    for (int t = 0; t < 4; ++t) {
+        sc[t] = float(scale[col + t]);
+        bs[t] = bias != nullptr ? float(bias[col + t]) : 0.0f;
+    }
 #pragma unroll
     for (int rb = 0; rb < RBA; ++rb)
 #pragma unroll
@@ -294,15 +298,15 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
             if (row < m) {
                 half4_t o;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) o[t] = _Float16(acc[rb][t][v] * sc[t]);
+                for (int t = 0; t < 4; ++t) o[t] = _Float16(fmaf(acc[rb][t][v], sc[t], bs[t]));
                 *reinterpret_cast<half4_t *>(c + int64_t(row) * n + col) = o;
             }
         }
 }
 
 template <int RB, int WM, int WN, int MIN_BLOCKS, int RBA, bool W_NK = false>
-void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n, int64_t lda,
-                  int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+void launch_cfg16(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k, int64_t n,
+                  int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     using Cfg = GemmW8Cfg16<RB, WM, WN>;
     const int tiles_m = int(cdiv(m, Cfg::kBM)), tiles_n = int(cdiv(n, Cfg::kBN));
     constexpr int kConcurrent = 32 * MIN_BLOCKS;  // workgroups an XCD (32 CUs) runs at a time
@@ -330,7 +334,7 @@ void launch_cfg16(const void *a, const void *w, const void *scale, void *c, int6
     allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA, W_NK>), Cfg::kLdsBytes);
     launch(gemm_w8a16_kernel16<RB, WM, WN, MIN_BLOCKS, RBA, W_NK>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const _Float16 *>(a), lda, static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale),
-           static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, split_unit, tail.parts, tail.max_tiles,
+           static_cast<const _Float16 *>(bias), static_cast<_Float16 *>(c), int(m), int(k), int(n), tiles_m, tiles_n, tiling.xm, tiling.xn, split_unit, tail.parts, tail.max_tiles,
            reinterpret_cast<float *>(ws.scratch), ws.counters);
 }
 
@@ -343,13 +347,13 @@ bool gemm_w8a16_supported(const void *a, const void *w, const void *c, int64_t m
            k * n < (int64_t(1) << 31) - (1 << 20) && (m * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
 }
 
-void gemm_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                       int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+void gemm_w8a16_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                       int64_t n, int64_t lda, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     // waves 128 x 64, workgroup tile 128 x 256; a matrix of at most 32 / 64 / 96 rows leaves the empty row blocks out
-    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
-    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
-    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
-    else launch_cfg16<8, 1, 4, 2, 8>(a, w, scale, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2>(a, w, scale, bias, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4>(a, w, scale, bias, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6>(a, w, scale, bias, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
+    else launch_cfg16<8, 1, 4, 2, 8>(a, w, scale, bias, c, m, k, n, lda, n, workspace, workspace_bytes, stream);
 }
 
 // The same kernel on a weight stored K-contiguous (w_nk[col * ldw + k]): 8-byte loads, so rows of w_nk 8-byte aligned.
@@ -360,12 +364,12 @@ bool gemm_w8a16_nk_supported(const void *a, const void *w, const void *c, int64_
            (m * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
 }
 
-void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                          int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
-    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
-    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
-    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
-    else launch_cfg16<8, 1, 4, 2, 8, true>(a, w, scale, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+void gemm_w8a16_nk_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                          int64_t n, int64_t lda, int64_t ldw, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    if (m <= 32) launch_cfg16<8, 1, 4, 2, 2, true>(a, w, scale, bias, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+    else if (m <= 64) launch_cfg16<8, 1, 4, 2, 4, true>(a, w, scale, bias, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+    else if (m <= 96) launch_cfg16<8, 1, 4, 2, 6, true>(a, w, scale, bias, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
+    else launch_cfg16<8, 1, 4, 2, 8, true>(a, w, scale, bias, c, m, k, n, lda, ldw, workspace, workspace_bytes, stream);
 }
 
 }  // namespace qmm

@@ -60,14 +60,25 @@ constexpr int kSkinnySpinLimit = 1 << 20;
 struct SkinnyScale {
     _Float16 one = _Float16(1.0f);                                                    // column tid % 256
     half4_t quad = {_Float16(1.0f), _Float16(1.0f), _Float16(1.0f), _Float16(1.0f)};  // columns 4 (tid % 64) .. + 3
+    _Float16 bias_one = _Float16(0.0f);                                               // added after the scale
+    half4_t bias_quad = {_Float16(0.0f), _Float16(0.0f), _Float16(0.0f), _Float16(0.0f)};
 };
-__device__ __forceinline__ SkinnyScale skinny_fetch_scale(const _Float16 *scale, int tile_col, int n, int m) {
+// `bias` may be null (no bias). 8-byte loads in the quad layout: scale and bias 8-byte aligned, n a multiple of 4.
+__device__ __forceinline__ SkinnyScale skinny_fetch_scale(const _Float16 *scale, const _Float16 *bias, int tile_col, int n, int m) {
     SkinnyScale s;
     const int tid = threadIdx.x;
     if (m <= 4) {
-        if (tile_col + (tid & 255) < n) s.one = scale[tile_col + (tid & 255)];
+        const int col = tile_col + (tid & 255);
+        if (col < n) {
+            s.one = scale[col];
+            if (bias != nullptr) s.bias_one = bias[col];
+        }
     } else {
-        if (tile_col + (tid & 63) * 4 < n) s.quad = *reinterpret_cast<const half4_t *>(scale + tile_col + (tid & 63) * 4);
+        const int col = tile_col + (tid & 63) * 4;
+        if (col < n) {
+            s.quad = *reinterpret_cast<const half4_t *>(scale + col);
+            if (bias != nullptr) s.bias_quad = *reinterpret_cast<const half4_t *>(bias + col);
+        }
     }
     return s;
 }
@@ -114,7 +125,7 @@ struct SkinnyTail {
     int m, n, row_first, col_in_tile;
     int64_t out_col;
     const float *red;
-    float scale[CW];
+    float scale[CW], bias[CW];
     OutT *c;
 
     struct Vals {
@@ -134,11 +145,11 @@ struct SkinnyTail {
     __device__ __forceinline__ void store(int row, const Vals &x) const {
         OutT *dst = c + int64_t(row) * n + out_col;
         if constexpr (CW == 1) {
-            dst[0] = skinny_to_out<OutT>(x.v[0] * scale[0]);
+            dst[0] = skinny_to_out<OutT>(fmaf(x.v[0], scale[0], bias[0]));
         } else {
             uint16_t h[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, skinny_to_out<OutT>(x.v[e] * scale[e]));
+            for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, skinny_to_out<OutT>(fmaf(x.v[e], scale[e], bias[e])));
             // 8 bytes at once when the row starts allow it (n a multiple of 4 is given, the base pointer may not be aligned)
             if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
                 *reinterpret_cast<uint2 *>(dst) = uint2{uint32_t(h[0]) | (uint32_t(h[1]) << 16), uint32_t(h[2]) | (uint32_t(h[3]) << 16)};
@@ -277,6 +288,7 @@ __device__ __forceinline__ void skinny_finish(const float4_t (&res)[16], int m, 
         tail.out_col = int64_t(tile) * kSkinnyTileN + tail.col_in_tile;
         tail.red = red;
         tail.scale[0] = float(col_scale.one);
+        tail.bias[0] = float(col_scale.bias_one);
         tail.c = c;
         if (tail.out_col < n && tail.row_first < m) tail.run(tile, split, splits, mailbox);
     } else {
@@ -288,7 +300,10 @@ __device__ __forceinline__ void skinny_finish(const float4_t (&res)[16], int m, 
         tail.out_col = int64_t(tile) * kSkinnyTileN + tail.col_in_tile;
         tail.red = red;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) tail.scale[e] = float(col_scale.quad[e]);
+        for (int e = 0; e < 4; ++e) {
+            tail.scale[e] = float(col_scale.quad[e]);
+            tail.bias[e] = float(col_scale.bias_quad[e]);
+        }
         tail.c = c;
         if (tail.out_col < n && tail.row_first < m) tail.run(tile, split, splits, mailbox);  // n is a multiple of 16: a quad is in or out as a whole
     }

@@ -154,7 +154,7 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(const u
             }
         }
     }
-    const SkinnyScale no_scale;  // all ones: the group scales are already in the totals
+    const SkinnyScale no_scale;  // ones and no bias: the group scales are already in the totals
     if (DT == HIDET_QMM_F16)
         skinny_finish<_Float16, kSkinnyWaves>(total, m, n, tile, split, splits, no_scale, reinterpret_cast<_Float16 *>(c), mailbox, red);
     else

@@ -33,7 +33,8 @@ struct SkinnyStep {
 template <bool ALIGNED_A, int WAVES, int RING>
 __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_kernel(const _Float16 *__restrict__ a, int64_t lda,
                                                                   const int8_t *__restrict__ w,
-                                                                  const _Float16 *__restrict__ scale, _Float16 *__restrict__ c,
+                                                                  const _Float16 *__restrict__ scale,
+                                                                  const _Float16 *__restrict__ bias, _Float16 *__restrict__ c,
                                                                   int m, int k, int n, int rows_per_block, int splits, int tiles,
                                                                   float *__restrict__ mailbox) {
     extern __shared__ float red[];  // [WAVES][m][kSkinnyRedStride]
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_kernel(const _Float16
 
     // the column factors this thread applies at the very end: fetched now, not looked at before then (a use here would
     // wait for the load before the first weight load is issued)
-    const SkinnyScale col_scale = skinny_fetch_scale(scale, tile_col, n, m);
+    const SkinnyScale col_scale = skinny_fetch_scale(scale, bias, tile_col, n, m);
 
     float4_t acc[16];
 #pragma unroll
@@ -142,21 +143,22 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_kernel(const _Float16
 // output element, serial K, fp32 accumulation.
 __global__ __launch_bounds__(256) void naive_w8a16_kernel(const _Float16 *__restrict__ a, int64_t lda,
                                                           const int8_t *__restrict__ w, const _Float16 *__restrict__ scale,
-                                                          _Float16 *__restrict__ c, int64_t m, int64_t k, int64_t n) {
+                                                          const _Float16 *__restrict__ bias, _Float16 *__restrict__ c, int64_t m,
+                                                          int64_t k, int64_t n) {
     const int64_t o = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (o >= m * n) return;
     const int64_t i = o / n, j = o - i * n;
     float acc = 0.f;
     for (int64_t kk = 0; kk < k; ++kk) acc += float(a[i * lda + kk]) * float(w[kk * n + j]);
-    c[o] = _Float16(acc * float(scale[j]));
+    c[o] = _Float16(fmaf(acc, float(scale[j]), bias != nullptr ? float(bias[j]) : 0.0f));
 }
 
 }  // namespace
 
-void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                         int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes, bool strict_workspace,
-                         hipStream_t stream) {
-    const bool fast = (n % 16 == 0) && aligned(w, 16) && aligned(scale, 8) && k > 0;  // 8-byte scale loads
+void skinny_w8a16_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                         int64_t n, int64_t lda, int parallel_k_parts, void *workspace, int64_t workspace_bytes,
+                         bool strict_workspace, hipStream_t stream) {
+    const bool fast = (n % 16 == 0) && aligned(w, 16) && aligned(scale, 8) && aligned(bias, 8) && k > 0;  // 8-byte scale and bias loads
     const int waves = 8;
     int rpb = 0, splits = 0, tiles = 0;
     const Workspace ws = split_workspace(workspace, workspace_bytes);
@@ -167,7 +169,8 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
     // a wave's K range is addressed with 31-bit offsets
     if (!fast || (int64_t(rpb) / waves + 160) * n >= (int64_t(1) << 31) - (1 << 20)) {
         launch(naive_w8a16_kernel, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, static_cast<const _Float16 *>(a), lda,
-               static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale), static_cast<_Float16 *>(c), m, k, n);
+               static_cast<const int8_t *>(w), static_cast<const _Float16 *>(scale), static_cast<const _Float16 *>(bias),
+               static_cast<_Float16 *>(c), m, k, n);
         return;
     }
     // 16-byte activation loads through a buffer descriptor: aligned rows, offsets below 2^31
@@ -181,7 +184,8 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, void *
         auto go = [&](auto kern) {
             if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16, waves)));  // the most any m needs
             launch(kern, dim3(grid), dim3(64 * waves), shmem, stream, ap, lda, static_cast<const int8_t *>(w),
-                   static_cast<const _Float16 *>(scale), cp, mt, int(k), int(n), rpb, splits, tiles, ws.mailbox);
+                   static_cast<const _Float16 *>(scale), static_cast<const _Float16 *>(bias), cp, mt, int(k), int(n), rpb, splits,
+                   tiles, ws.mailbox);
         };
         if (aligned_a) go(skinny_w8a16_kernel<true, 8, 1>);
         else go(skinny_w8a16_kernel<false, 8, 1>);

@@ -25,8 +25,8 @@ namespace {
 template <bool ALIGNED_A, bool FULL, int WAVES, bool STAGE = false>
 __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Float16 *__restrict__ a, int64_t lda,
                                                               const int8_t *__restrict__ w, int64_t ldw,
-                                                              const _Float16 *__restrict__ scale, _Float16 *__restrict__ c,
-                                                              int m, int k, int n) {
+                                                              const _Float16 *__restrict__ scale, const _Float16 *__restrict__ bias,
+                                                              _Float16 *__restrict__ c, int m, int k, int n) {
     __shared__ float red[WAVES][16][17];
     constexpr int kNkDepth = FULL ? 8 : 4;  // 128-deep steps per trip of the outer loop
     // STAGE (FULL with aligned activations, more than two rows): a wave fetches its 16 x 128 activation block of a step
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
         float v = 0.f;
 #pragma unroll
         for (int p = 0; p < WAVES; ++p) v += red[p][row][cn];
-        c[int64_t(row) * n + n0 + cn] = _Float16(v * float(scale[n0 + cn]));
+        c[int64_t(row) * n + n0 + cn] = _Float16(fmaf(v, float(scale[n0 + cn]), bias != nullptr ? float(bias[n0 + cn]) : 0.0f));
     }
 }
 
@@ -156,6 +156,7 @@ template <int CG, int WAVES, int DEPTH>
 __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_wide_kernel(const _Float16 *__restrict__ a, int64_t lda,
                                                                           const int8_t *__restrict__ w, int64_t ldw,
                                                                           const _Float16 *__restrict__ scale,
+                                                                          const _Float16 *__restrict__ bias,
                                                                           _Float16 *__restrict__ c, int m, int k, int n) {
     __shared__ float red[WAVES][CG][16][17];
     __shared__ uint4 stage[WAVES][2][16 * 17];  // per wave: activation block of a step, see the kernel above
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_wide_kernel(const 
             float v = 0.f;
 #pragma unroll
             for (int p = 0; p < WAVES; ++p) v += red[p][g][row][cn];
-            c[int64_t(row) * n + col] = _Float16(v * float(scale[col]));
+            c[int64_t(row) * n + col] = _Float16(fmaf(v, float(scale[col]), bias != nullptr ? float(bias[col]) : 0.0f));
         }
     }
 }
@@ -255,8 +256,8 @@ bool skinny_w8a16_nk_supported(const void *w, int64_t k, int64_t ldw) {
 
 // Any M: 16 rows per pass, every pass streams the weights again (beyond a few passes the [K, N] layout and its MFMA
 // GEMM are the better choice).
-void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, void *c, int64_t m, int64_t k, int64_t n,
-                            int64_t lda, int64_t ldw, hipStream_t stream) {
+void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, const void *bias, void *c, int64_t m, int64_t k,
+                            int64_t n, int64_t lda, int64_t ldw, hipStream_t stream) {
     const bool aligned_a = (lda % 8 == 0) && aligned(a, 16);
     const dim3 grid(uint32_t(cdiv(n, 16)));
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
@@ -265,13 +266,14 @@ void skinny_w8a16_nk_launch(const void *a, const void *w, const void *scale, voi
         _Float16 *cp = static_cast<_Float16 *>(c) + m0 * n;
         auto go = [&](auto kern, int waves) {
             launch(kern, grid, dim3(64 * waves), 0, stream, ap, lda, static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale),
-                   cp, mt, int(k), int(n));
+                   static_cast<const _Float16 *>(bias), cp, mt, int(k), int(n));
         };
         const bool full = k % 128 == 0;
         // more than 8 rows, a wide matrix and a long K: 32 columns per workgroup, the activation rows are read half as often
         if (full && aligned_a && mt > 8 && cdiv(n, 32) >= 256 && k >= 8192) {
             launch(skinny_w8a16_nk_wide_kernel<2, 8, 4>, dim3(uint32_t(cdiv(n, 32))), dim3(512), 0, stream, ap, lda,
-                   static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale), cp, mt, int(k), int(n));
+                   static_cast<const int8_t *>(w), ldw, static_cast<const _Float16 *>(scale), static_cast<const _Float16 *>(bias), cp,
+                   mt, int(k), int(n));
             continue;
         }
         // few column tiles: eight waves per workgroup keep enough loads in flight on each compute unit

@@ -41,6 +41,8 @@ SIGNATURES = {
     'hidet_symmetric_quantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _i64, _vp]),
     'hidet_symmetric_dequantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     'hidet_symmetric_quant_matmul_f16_i8': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
+    'hidet_symmetric_quant_matmul_f16_i8_bias': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
+    'hidet_symmetric_quant_matmul_f16_i8_nk_bias': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     'hidet_qmm_static_scratch_bytes': (_i64, []),
     'hidet_symmetric_quant_matmul_f16_i8_static': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp]),
     'hidet_symmetric_quant_matmul_f16_i8_nk': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),

@@ -1,6 +1,6 @@
 """symmetric_quant_matmul with the reference's signature, checks and error texts
 (python/hidet/graph/ops/quant/matmul.py:24-93), executed by `hidet_symmetric_quant_matmul_f16_i8`."""
-from typing import List
+from typing import List, Optional
 
 import torch
 
@@ -79,11 +79,21 @@ def _row_major(weight: torch.Tensor) -> torch.Tensor:
     return weight.contiguous()
 
 
-def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parallel_k_parts: int = 0) -> torch.Tensor:
+def _check_bias(bias: torch.Tensor, n: int) -> torch.Tensor:
+    if bias.dtype != torch.float16 or bias.dim() != 1 or bias.shape[0] != n:
+        raise ValueError('bias must be a float16 vector of {} elements, got {} {}'.format(n, bias.dtype, list(bias.shape)))
+    return bias.contiguous()
+
+
+def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parallel_k_parts: int = 0,
+              bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """c[..., M, N] on the GPU.  Leading axes of `a` are folded into M: the weight is 2-D, so broadcasting
-    over them is the same as one tall matmul."""
+    over them is the same as one tall matmul.  `bias` (float16 [N]) is added in the kernel's epilogue."""
     ffi.require_gpu(a, weight, scale)
     k, n = weight.shape
+    if bias is not None:
+        ffi.require_gpu(bias)
+        bias = _check_bias(bias, n)
     a2 = a.reshape(-1, k)
     if a2.stride(-1) != 1 or (a2.shape[0] > 1 and a2.stride(0) < k):
         a2 = a2.contiguous()
@@ -100,19 +110,30 @@ def run_w8a16(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor, parall
                                        and (n - 1) * weight.stride(1) + k < (1 << 31) - (1 << 20)
                                        and (m * lda + k) * 2 < (1 << 31) - (1 << 20)))):
         ws = ffi.workspace(a.device)
-        ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a2, weight, scale, c, m, k, n, lda, weight.stride(1), ws, ws.numel(),
-                 ffi.current_stream(a.device))
+        if bias is None:
+            ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', a2, weight, scale, c, m, k, n, lda, weight.stride(1), ws, ws.numel(),
+                     ffi.current_stream(a.device))
+        else:
+            ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk_bias', a2, weight, scale, bias, c, m, k, n, lda, weight.stride(1), ws,
+                     ws.numel(), ffi.current_stream(a.device))
         return c.reshape(tuple(a.shape[:-1]) + (n,))
     weight = _row_major(weight)
     ws = ffi.workspace(a.device)
-    ffi.call('hidet_symmetric_quant_matmul_f16_i8', a2, weight, scale, c, m, k, n, lda, int(parallel_k_parts), ws,
-             ws.numel(), ffi.current_stream(a.device))
+    if bias is None:
+        ffi.call('hidet_symmetric_quant_matmul_f16_i8', a2, weight, scale, c, m, k, n, lda, int(parallel_k_parts), ws,
+                 ws.numel(), ffi.current_stream(a.device))
+    else:
+        ffi.call('hidet_symmetric_quant_matmul_f16_i8_bias', a2, weight, scale, bias, c, m, k, n, lda, int(parallel_k_parts), ws,
+                 ws.numel(), ffi.current_stream(a.device))
     return c.reshape(tuple(a.shape[:-1]) + (n,))
 
 
 class SymmetricQuantizedMatmulOp(Operator):
-    def __init__(self, a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor):
+    def __init__(self, a: torch.Tensor, b: torch.Tensor, scale: torch.Tensor, bias: Optional[torch.Tensor] = None):
         task = SymmetricQuantizedMatmulTask(input_like(a, 'a'), input_like(b, 'b'), input_like(scale, 'scale'))
+        if bias is not None:
+            _check_bias(bias, b.shape[1])
+        self.bias = bias
         super().__init__(inputs=[a, b, scale], attributes={}, task=task)
 
     def run(self) -> List[torch.Tensor]:
@@ -120,7 +141,7 @@ class SymmetricQuantizedMatmulOp(Operator):
 
         a, b, scale = self.inputs
         parts = resolve_parallel_k_parts(option.get_parallel_k(), a, b)
-        return [run_w8a16(a, b, scale, parts)]
+        return [run_w8a16(a, b, scale, parts, self.bias)]
 
 
 # Operand signatures (shapes and dtypes) that have passed every check once.  A decode loop calls the operator with the same
@@ -129,13 +150,18 @@ class SymmetricQuantizedMatmulOp(Operator):
 _VALIDATED = set()
 
 
-def symmetric_quant_matmul(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-    signature = (a.shape, a.dtype, weight.shape, weight.dtype, scale.shape, scale.dtype)
+def symmetric_quant_matmul(a: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor,
+                           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The reference's operator (python/hidet/graph/ops/quant/matmul.py:83-93).  `bias`, which the reference's signature
+    does not have, is the fused form of the epilogue its template admits (matmul_f16_i8.py:95-99): a float16 [N] vector
+    added to the fp32 result before the one rounding to float16."""
+    signature = (a.shape, a.dtype, weight.shape, weight.dtype, scale.shape, scale.dtype,
+                 None if bias is None else (bias.shape, bias.dtype))
     if signature in _VALIDATED:
         from .resolve import resolve_parallel_k_parts
 
-        return run_w8a16(a, weight, scale, resolve_parallel_k_parts(option.get_parallel_k(), a, weight))
+        return run_w8a16(a, weight, scale, resolve_parallel_k_parts(option.get_parallel_k(), a, weight), bias)
     check_matmul_args(a, weight)
-    out = SymmetricQuantizedMatmulOp(a, weight, scale).outputs[0]
+    out = SymmetricQuantizedMatmulOp(a, weight, scale, bias).outputs[0]
     _VALIDATED.add(signature)
     return out

@@ -196,6 +196,49 @@ class SymmetricQuantizeMatmulFused(SubgraphRewriteRule):
         return count
 
 
+class SymmetricQuantizeMatmulBiasFused(SubgraphRewriteRule):
+    """add(symmetric_quant_matmul(x, wq, scale), bias) => symmetric_quant_matmul(x, wq, scale, bias) for a constant float16
+    bias of one element per output column: the bias of an nn.Linear rides in the kernel's epilogue instead of a separate
+    element-wise launch per layer. The reference gets the same effect from its fusion pass, which folds the add into the
+    template's epilogue (matmul_f16_i8.py:95-99, allow_epilogue); there is no rule of this name there."""
+
+    def __init__(self):
+        super().__init__('add(fused_matmulf16(x, wq, scale), bias) => fused_matmulf16(x, wq, scale, bias)')
+
+    def apply(self, gm: fx.GraphModule, ctx: PassContext) -> int:
+        import operator as py_operator
+
+        quant = _quant_ops()
+        count = 0
+        for node in list(gm.graph.nodes):
+            if not (node.op == 'call_function' and node.target in (torch.add, py_operator.add) and len(node.args) == 2
+                    and not node.kwargs):
+                continue
+            for mm, other in ((node.args[0], node.args[1]), (node.args[1], node.args[0])):
+                if not (isinstance(mm, fx.Node) and mm.op == 'call_function' and mm.target is quant.symmetric_quant_matmul
+                        and len(mm.args) == 3 and not mm.kwargs and len(mm.users) == 1 and isinstance(other, fx.Node)):
+                    continue
+                bias = constant_of(gm, other)
+                wq = constant_of(gm, mm.args[1])
+                if bias is None or wq is None or bias.dim() != 1 or bias.shape[0] != wq.shape[1] or bias.dtype != torch.float16:
+                    continue
+                with gm.graph.inserting_before(node):
+                    out = gm.graph.call_function(quant.symmetric_quant_matmul, tuple(mm.args) + (other,))
+                out.meta = dict(node.meta)
+                node.replace_all_uses_with(out)
+                gm.graph.erase_node(node)
+                gm.graph.erase_node(mm)
+                count += 1
+                break
+        return count
+
+
 def matmul_specialization_rules() -> List[SubgraphRewriteRule]:
     """Rules that replace generic sub-graphs by fused operators where those apply (linear.py:127-129)."""
     return [SymmetricQuantizeMatmulFused()]
+
+
+def epilogue_fusion_rules() -> List[SubgraphRewriteRule]:
+    """What the reference leaves to its operator-fusion pass, which runs after the quantize rules: here the quantize pass
+    applies these once the context's own rules are done."""
+    return [SymmetricQuantizeMatmulBiasFused()]

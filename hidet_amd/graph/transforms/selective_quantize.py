@@ -7,8 +7,13 @@ from .base import GraphPass, PassContext
 
 class SelectiveQuantizePass(GraphPass):
     def process_graph(self, gm: fx.GraphModule) -> fx.GraphModule:
+        from .graph_patterns.quant.linear import epilogue_fusion_rules
+
         ctx = PassContext.current()
-        for rule in ctx.configs['quantize_patterns']:
+        rules = list(ctx.configs['quantize_patterns'])
+        if rules:  # the fused operators those rules leave behind take their layer's bias into the epilogue
+            rules += epilogue_fusion_rules()
+        for rule in rules:
             count = rule.apply(gm, ctx)
             ctx.rewrites.append((rule.name, count))
             if ctx.configs['verbose']:

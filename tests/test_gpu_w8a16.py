@@ -99,6 +99,29 @@ def test_split_k_parts_api_and_hints():
         assert O.max_rel_err(host(c), host(base)) < 1e-3
 
 
+@pytest.mark.parametrize('m,k,n,layout', [(1, 4096, 11008, 'kn'), (3, 1024, 768, 'kn'), (8, 2048, 4096, 'kn'), (16, 512, 256, 'kn'),
+                                          (12, 512, 8200, 'kn'), (40, 2048, 520, 'kn'), (300, 512, 1100, 'kn'), (2, 100, 40, 'kn'),
+                                          (1, 4096, 1024, 'nk'), (16, 1024, 512, 'nk'), (40, 2048, 520, 'nk'), (12, 8192, 8192, 'nk')])
+def test_bias_in_the_epilogue_exact(m, k, n, layout):
+    # c = acc * scale + bias with one rounding: integer operands, power-of-two scales and a bias of small multiples of
+    # 2^-10 make every step exact in fp32; every kernel family that has the epilogue (both tail layouts of the
+    # bandwidth-bound kernel, the MFMA GEMM, the element-wise fallback, the kernels for K-contiguous weights)
+    announce('w8a16 bias', m, k, n, layout)
+    a, q, s = _int_case(m * 7 + n, m, k, n)
+    rng = np.random.default_rng(n)
+    b = (rng.integers(-64, 65, n) / 1024.0).astype(np.float16)
+    want = (a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :] + b.astype(np.float64)[None, :]
+    tq = dev(q)
+    if layout == 'nk':
+        tq = quant.to_decode_layout(tq)
+    got = host(quant.symmetric_quant_matmul(dev(a), tq, dev(s), dev(b)))
+    assert np.array_equal(got, want.astype(np.float32).astype(np.float16))
+    plain = host(quant.symmetric_quant_matmul(dev(a), tq, dev(s)))  # the same call without bias is unchanged
+    assert np.array_equal(plain, (want - b.astype(np.float64)[None, :]).astype(np.float32).astype(np.float16))
+    with pytest.raises(ValueError, match='bias must be'):
+        quant.symmetric_quant_matmul(dev(a), tq, dev(s), dev(b[:-1]))
+
+
 def test_parallel_k_search():
     # hidet.option.parallel_k('search') (reference resolve.py:53-92): the candidates are timed on the GPU, the winner is
     # one of them (or 0, the library's own plan), is remembered per shape, and the result equals the unsplit one

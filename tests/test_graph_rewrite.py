@@ -34,12 +34,16 @@ def cpu_ops(monkeypatch):
         calls['dequantize'] += 1
         return torch.from_numpy(O.symmetric_dequantize(wq.numpy(), scale.numpy(), dims=dims))
 
-    def symmetric_quant_matmul(a, wq, scale):
+    def symmetric_quant_matmul(a, wq, scale, bias=None):
         calls['matmul'] += 1
         assert a.dtype == torch.float16 and wq.dtype == torch.int8 and scale.dtype == torch.float16
         a2 = a.reshape(-1, a.shape[-1]).numpy()
-        out = O.symmetric_quant_matmul(a2, wq.numpy(), scale.numpy())
-        return torch.from_numpy(out).reshape(*a.shape[:-1], wq.shape[1])
+        out = torch.from_numpy(O.symmetric_quant_matmul(a2, wq.numpy(), scale.numpy())).reshape(*a.shape[:-1], wq.shape[1])
+        if bias is not None:
+            calls['bias'] = calls.get('bias', 0) + 1
+            assert bias.dtype == torch.float16 and tuple(bias.shape) == (wq.shape[1],)
+            out = out + bias
+        return out
 
     monkeypatch.setattr(quant_ops, 'symmetric_quantize', symmetric_quantize)
     monkeypatch.setattr(quant_ops, 'symmetric_dequantize', symmetric_dequantize)
@@ -105,6 +109,31 @@ def test_linear_modules_become_fused_operator(cpu_ops):
     got = gm(x.half())
     assert got.dtype == torch.float16 and cpu_ops['matmul'] == 2
     assert O.max_rel_err(got.float().numpy(), want.detach().numpy()) < 3e-2
+
+
+def test_bias_moves_into_the_fused_operator(cpu_ops):
+    # nn.Linear with bias: matmul + add becomes one call of the fused operator with the bias as its fourth argument
+    torch.manual_seed(5)
+    model = Mlp(bias=True).eval()
+    x = torch.randn(2, 7, 32)
+    want = model(x)
+    with PassContext() as ctx:
+        ctx.set_precision('int8')
+        gm = quantize_module(model, ctx)
+        assert ctx.rewrites[-1][1] == 2  # the epilogue rule ran last and fused both layers
+    targets = _targets(gm)
+    assert targets.count(quant_ops.symmetric_quant_matmul) == 2 and torch.add not in targets
+    mm_nodes = [n for n in gm.graph.nodes if n.op == 'call_function' and n.target is quant_ops.symmetric_quant_matmul]
+    assert all(len(n.args) == 4 for n in mm_nodes)
+    got = gm(x.half())
+    assert cpu_ops.get('bias') == 2
+    assert O.max_rel_err(got.float().numpy(), want.detach().numpy()) < 3e-2
+    # without bias nothing changes; a bias that is not a constant vector of N elements stays an add
+    with PassContext() as ctx:
+        ctx.set_precision('int8')
+        gm2 = quantize_module(Mlp(bias=False).eval(), ctx)
+        assert ctx.rewrites[-1][1] == 0
+    assert all(len(n.args) == 3 for n in gm2.graph.nodes if n.op == 'call_function' and n.target is quant_ops.symmetric_quant_matmul)
 
 
 def test_quantize_module_leaves_the_source_model_untouched(cpu_ops):
