@@ -122,6 +122,23 @@ def test_bias_in_the_epilogue_exact(m, k, n, layout):
         quant.symmetric_quant_matmul(dev(a), tq, dev(s), dev(b[:-1]))
 
 
+@pytest.mark.parametrize('m,k,n,parts', [(2, 8192, 16384, 32), (16, 4096, 8192, 16), (1, 16384, 4096, 64)])
+def test_more_workgroups_than_the_chip_holds(m, k, n, parts):
+    # a forced K split far beyond one round (2048 / 512 / 1024 workgroups of 8 waves on 256 CUs): the workgroup that
+    # collects a column tile's partial sums is the last of that tile in launch order, so everything it waits for was
+    # started before it; the result is exact, twice in a row (the mailbox is clean again after the first call)
+    announce('w8a16 oversubscribed', m, k, n, parts)
+    a, q, s = _int_case(m + k, m, k, n)
+    want = ((a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :])
+    ta, tq, ts = dev(a), dev(q), dev(s)
+    for _ in range(2):
+        c = torch.full((m, n), float('nan'), dtype=torch.float16, device='cuda')
+        ws = hidet_amd.ffi.workspace(ta.device)
+        hidet_amd.ffi.call('hidet_symmetric_quant_matmul_f16_i8', ta, tq, ts, c, m, k, n, k, parts, ws, ws.numel(),
+                           hidet_amd.ffi.current_stream(ta.device))
+        assert np.array_equal(host(c), want.astype(np.float32).astype(np.float16))
+
+
 def test_parallel_k_search():
     # hidet.option.parallel_k('search') (reference resolve.py:53-92): the candidates are timed on the GPU, the winner is
     # one of them (or 0, the library's own plan), is remembered per shape, and the result equals the unsplit one
