@@ -7,7 +7,14 @@
 namespace qmm {
 
 constexpr int kSkinnyTileN = 256;
-constexpr int kSkinnyRedStride = 272;  // 16 lanes x 17 floats: conflict-free LDS writes
+// LDS reduction tile: one row of 256 floats per (wave, activation row), 1040 bytes apart, as 64 chunks of 16 bytes. The
+// chunk of columns 4c .. 4c+3 sits at position skinny_red_chunk(c). A lane (g, cl) of the main loop writes the four
+// chunks 4cl .. 4cl+3 of rows 4g .. 4g+3 with 16-byte stores: the row pitch puts the four g of an instruction into
+// different quarters of the 64 banks (4 rows = 16 x 256 + 64 bytes) and the permutation spreads the four lanes that
+// share a quarter over its four 16-byte slots, so an instruction takes the four passes its 1 KiB needs and no more.
+// Readers fetch whole chunks (or single floats of them) of consecutive columns: every bank once per 256 bytes.
+constexpr int kSkinnyRedStride = 260;  // floats
+__device__ __forceinline__ int skinny_red_chunk(int c) { return (c & ~3) | ((c ^ (c >> 4)) & 3); }
 
 inline size_t skinny_lds_bytes(int m, int waves) { return size_t(waves) * m * kSkinnyRedStride * sizeof(float); }
 
@@ -132,14 +139,20 @@ struct SkinnyTail {
         float v[CW];
     };
     __device__ __forceinline__ Vals own(int row) const {
-        const float *src = red + row * kSkinnyRedStride + col_in_tile + (col_in_tile >> 4);  // CW columns never straddle 16
+        const float *src = red + row * kSkinnyRedStride + skinny_red_chunk(col_in_tile >> 2) * 4 + (col_in_tile & 3);  // CW columns never straddle a chunk
         Vals r;
 #pragma unroll
         for (int e = 0; e < CW; ++e) r.v[e] = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < WAVES; ++wv)
+        for (int wv = 0; wv < WAVES; ++wv) {
+            if constexpr (CW == 4) {
+                const float4_t q = *reinterpret_cast<const float4_t *>(src + wv * m * kSkinnyRedStride);
 #pragma unroll
-            for (int e = 0; e < CW; ++e) r.v[e] += src[wv * m * kSkinnyRedStride + e];
+                for (int e = 0; e < 4; ++e) r.v[e] += q[e];
+            } else {
+                r.v[0] += src[wv * m * kSkinnyRedStride];
+            }
+        }
         return r;
     }
     __device__ __forceinline__ void store(int row, const Vals &x) const {
@@ -272,9 +285,11 @@ __device__ __forceinline__ void skinny_finish(const float4_t (&res)[16], int m, 
     for (int v = 0; v < 4; ++v) {
         const int row = 4 * g + v;
         if (row < m) {
-            float *dst = red + (wave * m + row) * kSkinnyRedStride + cl * 17;
+            float *dst = red + (wave * m + row) * kSkinnyRedStride;
 #pragma unroll
-            for (int t = 0; t < 16; ++t) dst[t] = res[t][v];
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<float4_t *>(dst + skinny_red_chunk(4 * cl + j) * 4) =
+                    float4_t{res[4 * j][v], res[4 * j + 1][v], res[4 * j + 2][v], res[4 * j + 3][v]};
         }
     }
     __syncthreads();
