@@ -262,6 +262,8 @@ def main():
     evs = [(lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()) for _ in range(RING)]
     durs = []
     for rep in range(9):
+        for i in range(RING - 4, RING):  # untimed: the pass starts behind a synchronisation, the timed region does not
+            launch(i, sptr)
         for i in range(RING):
             lib.hidet_qmm_arm_timing(evs[i][0], evs[i][1])
             launch(i, sptr)
@@ -360,6 +362,8 @@ def main():
         d = []
         for r0 in range(0, reps, 16):
             nb = min(16, reps - r0)
+            for j in range(2):  # untimed: a batch starts behind a synchronisation, a decode step does not
+                fn(r0 + nb - 1 - j)
             for j in range(nb):
                 lib.hidet_qmm_arm_timing(pairs[j][0], pairs[j][1])
                 fn(r0 + j)
@@ -405,6 +409,15 @@ def main():
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ad, ws[r % RING].view(K, N), sd, cd, 1, N, K, N, N,
                                       None, 0, sptr), 48, 16)
     others['w8a16_gemv_down_proj_k11008_n4096_k_contiguous_weights'] = hbm_entry(us, K * N + 2 * K + 2 * N + 2 * K)
+    # the same GEMV on the first 256 ... 2048 rows of the ring's matrices (and all 4096): time against K at N = 11008 separates
+    # what a launch costs whatever it reads from what its bytes cost
+    sweep = {}
+    for kk in (256, 1024, 2048, 4096):
+        ak = a[:, :kk].contiguous()
+        us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ak, ws[r % RING], ss[0], cu, 1, kk, N, kk, 0,
+                                          work, work.numel(), sptr), 48, 16)
+        sweep['k{}'.format(kk)] = round(us, 2)
+    others['w8a16_gemv_n11008_us_against_k'] = sweep
     # the same GEMV kernel on a matrix five times the size (not a benchmark configuration: it shows how much of the headline
     # figure is the fixed cost of one launch and one cross-workgroup exchange)
     wl = [torch.randint(-127, 128, (8192, 28672), device=device, dtype=torch.int8) for _ in range(3)]  # 3 x 235 MB > LLC
@@ -503,7 +516,7 @@ def main():
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': GEMV_MEASURED_TRAFFIC_BYTES,
                      'traffic_source': GEMV_TRAFFIC_PROFILE, 'algorithmic_bytes': GEMV_BYTES,
-                     'duration_of': 'every launch of the ring, launched back to back, begin/end of its own dispatch',
+                     'duration_of': 'every launch of the ring, launched back to back behind four untimed launches, begin/end of its own dispatch',
                      'kernel': 'skinny_w8a16_kernel', 'kernel_us_mean': round(kernel_us, 3),
                      'kernel_us_min': round(float(durs.min()), 3), 'kernel_us_p50': round(float(np.median(durs)), 3),
                      'launches_timed': int(durs.size)},
