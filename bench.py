@@ -34,7 +34,7 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0
 # HBM bytes one GEMV launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over the --pmc-calibration
 # run of this file, each scaled by what the same counter reads for a 64 MiB device copy. The figure is a record of that
 # profile, not measured in this run: it is reported together with the name of the summary it was taken from.
-GEMV_MEASURED_TRAFFIC_BYTES = 45.81e6
+GEMV_MEASURED_TRAFFIC_BYTES = 45.83e6
 GEMV_TRAFFIC_PROFILE = 'profiles/skinny_w8a16_gemv_m1_k4096_n11008_hbm_traffic.md'
 K, N = 4096, 11008
 RING = 16
