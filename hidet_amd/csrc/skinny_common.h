@@ -43,9 +43,9 @@ __device__ __forceinline__ bool skinny_tile_of_block(int splits, int tiles, int 
 // the split-K exchange through the mailbox.
 //
 // res[t][v] is this lane's partial sum for output row 4 * (lane / 16) + v and column tile * 256 + (lane % 16) * 16 + t.
-// `red` is dynamic LDS of skinny_lds_bytes(m, WAVES). col_scale points at the factors of the tile's 256 columns (or is
-// null); the factors a thread needs are fetched before the caller's main loop would be ideal, but they come from the
-// cache by the time the tail runs: the caller touches them early (skinny_prefetch_scale).
+// `red` is dynamic LDS of skinny_lds_bytes(m, WAVES). col_scale holds the column factors and biases this thread applies
+// to its outputs (SkinnyScale: the caller fetches them with skinny_fetch_scale before its main loop, so that no load
+// sits between the last weight and the output).
 //
 // Who does what in the tail: with up to 4 rows thread tid owns column tid % 256 of rows tid / 256, tid / 256 + WAVES / 4,
 // ... (one dword per access, four waves per row); with more rows it owns columns 4 (tid % 64) .. + 3 of rows tid / 64,
