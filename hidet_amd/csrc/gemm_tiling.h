@@ -190,6 +190,9 @@ __device__ __forceinline__ bool gemm_k_split_fixup(float4_t (&acc)[R][T], const 
                                                    ((item.part * R + r) * T + t) * (THREADS * 16), kAgentScope);
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // vmcnt(0): every store of this lane has been acknowledged
+    // The stores above write through (agent scope) and are complete; the fence tells the compiler, too, that nothing
+    // may move across this point (at workgroup scope it emits no cache operation)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t old = __hip_atomic_fetch_add(&counters[item.slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -198,6 +201,7 @@ __device__ __forceinline__ bool gemm_k_split_fixup(float4_t (&acc)[R][T], const 
     }
     __syncthreads();
     if (!*flag) return false;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the reads below stay below (they bypass the L1 themselves)
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
