@@ -220,3 +220,29 @@ def test_fp8_scaled_operands_broadcast():
     a3, b3, sa3, sb3, head = F8.scaled_operands(a, b5, sa, sb5)
     assert head == (2, 3) and a3.shape[0] == 6 and b3.shape[0] == 6 and sa3.shape[0] == 6 and sb3.shape[0] == 6
     assert torch.equal(b3[4], b5[1]) and torch.equal(a3[4], a[1, 1])
+
+
+def test_task_library_calling_form(tmp_path):
+    # the reference's compiled-task interface for one concrete task: hidet_launch_0 / hidet_get_input_shape /
+    # hidet_get_output_shape in a lib.so of the task directory, and meta.json (python/hidet/drivers/build_task.py:63-140,
+    # python/hidet/runtime/compiled_task.py:31-39, 68-79)
+    import json
+    from hidet_amd.drivers import build_task_library
+    so = build_task_library(str(tmp_path), 3, 128, 64)
+    lib = ctypes.CDLL(so)
+    for name in ('hidet_launch_0', 'hidet_get_input_shape', 'hidet_get_output_shape', 'hidet_qmm_task_set_stream'):
+        assert hasattr(lib, name)
+    dims = (ctypes.c_int32 * 4)(-1, -1, -1, -1)
+    want = {0: [3, 128], 1: [128, 64], 2: [64]}
+    for idx, shape in want.items():
+        for j in range(4):
+            dims[j] = -1
+        lib.hidet_get_input_shape(idx, dims)
+        assert list(dims)[:len(shape)] == shape and all(d == -1 for d in list(dims)[len(shape):])
+    lib.hidet_get_output_shape(0, dims)
+    assert list(dims)[:2] == [3, 64]
+    meta = json.load(open(tmp_path / 'meta.json'))
+    assert meta['num_candidates'] == 1 and [i['shape'] for i in meta['inputs']] == [[3, 128], [128, 64], [64]]
+    assert meta['outputs'][0]['shape'] == [3, 64] and meta['name'] == 'symmetric_quantized_matmul'
+    with pytest.raises(ValueError):
+        build_task_library(str(tmp_path), 0, 128, 64)

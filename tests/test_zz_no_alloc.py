@@ -97,3 +97,25 @@ def test_static_scratch_rejects_oversized_split():
     a2, q2, s2 = _case(3, 1, 1024, 512)
     got = host(_static(dev(a2), dev(q2), dev(s2)))
     assert O.max_rel_err(got, clib.quant_matmul_f32acc(a2, q2, s2)) <= 1e-2
+
+
+def test_task_library_launch_matches_the_operator(tmp_path):
+    # hidet_launch_0(a, weight, scale, c) of a generated task library (pointers only, shapes fixed at build time) runs the
+    # entry point that needs no workspace; same result as the operator, on the stream set for the task
+    import ctypes
+    from hidet_amd.drivers import build_task_library
+    from hidet_amd.graph.ops import quant
+    m, k, n = 2, 2048, 1024
+    announce('task library', m, k, n)
+    a, q, s = _case(21, m, k, n)
+    da, dq, ds = dev(a), dev(q), dev(s)
+    lib = ctypes.CDLL(build_task_library(str(tmp_path), m, k, n))
+    lib.hidet_launch_0.argtypes = [ctypes.c_void_p] * 4
+    lib.hidet_qmm_task_set_stream.argtypes = [ctypes.c_void_p]
+    c = torch.full((m, n), float('nan'), dtype=torch.float16, device='cuda')
+    lib.hidet_qmm_task_set_stream(ffi.current_stream(da.device))
+    lib.hidet_launch_0(da.data_ptr(), dq.data_ptr(), ds.data_ptr(), c.data_ptr())
+    assert ffi.get_last_error() is None
+    want = quant.symmetric_quant_matmul(da, dq, ds)
+    assert torch.equal(c, want)
+    assert O.max_rel_err(host(c), clib.quant_matmul_f32acc(a, q, s)) <= 1e-2
