@@ -35,11 +35,10 @@ void w8a16_dispatch(const void *a, const void *w, const void *scale, const void 
     QMM_CHECK(aligned(a, 2) && aligned(scale, 2) && aligned(c, 2) && aligned(bias, 2), "float16 tensors must be 2-byte aligned");
     // Up to 16 rows one pass of the bandwidth-bound kernel serves; beyond that every 16 rows would cost another pass
     // over the weights, and the MFMA GEMM with its K split and its empty row blocks left out takes over (K=4096, N=11008,
-    // weights from HBM: 17 us at M=17..32, 20 us at M=64, 29 us at M=128). From 9 rows on the GEMM is already ahead when
-    // the output is wide enough for its 256-column tiles to fill the chip (N=11008: 16.0 against 18.4 us; N=4096: 13.6
-    // against 13.4 us), unless the caller asked for a specific K split of the bandwidth-bound kernel.
-    const bool wide = cdiv(n, 256) >= 32;
-    if ((m > 16 || (m > 8 && wide && parallel_k_parts == 0)) && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
+    // weights from HBM: 17 us at M=17..32, 20 us at M=64, 29 us at M=128). For 9 to 16 rows the bandwidth-bound kernel is
+    // ahead of the GEMM on every shape measured (4096 x 11008: 13.5 - 14.1 against 16.5 us; 8192 x 8192: 16.9 - 18.2
+    // against 22.4; 8192 x 28672: 42.6 - 43.8 against 49).
+    if (m > 16 && k > 0 && gemm_w8a16_supported(a, w, c, m, k, n, lda))
         gemm_w8a16_launch(a, w, scale, bias, c, m, k, n, lda, workspace, workspace_bytes, stream);
     else
         skinny_w8a16_launch(a, w, scale, bias, c, m, k, n, lda, parallel_k_parts, workspace, workspace_bytes, strict_workspace,

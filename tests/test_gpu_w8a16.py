@@ -31,7 +31,7 @@ def _int_case(seed, m, k, n):
 
 @pytest.mark.parametrize('m,k,n', [(1, 256, 256), (1, 4096, 512), (3, 1024, 768), (16, 512, 256), (7, 96, 48),
                                    (1, 40, 16), (2, 8, 16), (1, 4096, 272), (16, 4096, 4096),
-                                   (9, 4096, 8192), (16, 1024, 11008), (12, 512, 8200)])  # wide outputs: 9+ rows take the MFMA GEMM
+                                   (9, 4096, 8192), (16, 1024, 11008), (12, 512, 8200)])  # 9 to 16 rows on wide outputs
 def test_exact_on_small_integers(m, k, n):
     # integer activations and codes with power-of-two scales: every product and partial sum is exact in
     # fp32, so any dropped row, wrong byte or lost K slice shows as a whole-number difference
