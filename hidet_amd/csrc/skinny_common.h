@@ -47,11 +47,13 @@ __device__ __forceinline__ bool skinny_tile_of_block(int splits, int tiles, int 
 // to its outputs (SkinnyScale: the caller fetches them with skinny_fetch_scale before its main loop, so that no load
 // sits between the last weight and the output).
 //
-// Who does what in the tail: with up to 4 rows thread tid owns column tid % 256 of rows tid / 256, tid / 256 + WAVES / 4,
-// ... (one dword per access, four waves per row); with more rows it owns columns 4 (tid % 64) .. + 3 of rows tid / 64,
+// Who does what in the tail: in the column layout thread tid owns column tid % 256 of rows tid / 256, tid / 256 + WAVES / 4,
+// ... (one dword per access, four waves per row); in the quad layout it owns columns 4 (tid % 64) .. + 3 of rows tid / 64,
 // tid / 64 + WAVES, ... (16 bytes per access, one wave per row). Either way every wave has work: the same bytes moved
 // by a single wave were measured 1 us slower per launch, and every batch of reads from the mailbox costs a round trip
-// to the memory side (1.5 to 2 us), so a thread wants all its reads in one batch of 16.
+// to the memory side (1.5 to 2 us), so a thread wants all its reads in one batch of 16. The column layout is the faster
+// one per byte (8 rows at 4096 x 11008: 12.9 against 13.3 us) and is used whenever its reads fit that one batch
+// (skinny_column_layout).
 //
 // Exchange: the mailbox holds one fp32 tile [m][256] per (column tile, K slice) and is all zero between launches. Every
 // slice but the last stores its tile (agent scope, +0.0 sent as -0.0, so a stored word is never zero) and is done: no
@@ -70,11 +72,21 @@ struct SkinnyScale {
     _Float16 bias_one = _Float16(0.0f);                                               // added after the scale
     half4_t bias_quad = {_Float16(0.0f), _Float16(0.0f), _Float16(0.0f), _Float16(0.0f)};
 };
+// Which of the tail's two thread layouts a launch uses: one column per thread (dwords, `waves / 4` rows at a time) while a
+// thread's reads of the exchange fit one batch of 16 - rows per thread x other slices, in the shapes collect<LG> has:
+// 4 x 4, 2 x 8 or 1 x 16 - and whenever nothing is exchanged and there are few rows; else four columns per thread.
+__device__ __forceinline__ bool skinny_column_layout(int m, int splits, int waves) {
+    const int row_groups = waves / 4, rows = (m + row_groups - 1) / row_groups, others = splits - 1;
+    if (others == 0) return m <= 4;
+    return (rows <= 4 && others <= 4) || (rows <= 2 && others <= 8) || (rows <= 1 && others <= 16);
+}
+
 // `bias` may be null (no bias). 8-byte loads in the quad layout: scale and bias 8-byte aligned, n a multiple of 4.
-__device__ __forceinline__ SkinnyScale skinny_fetch_scale(const _Float16 *scale, const _Float16 *bias, int tile_col, int n, int m) {
+__device__ __forceinline__ SkinnyScale skinny_fetch_scale(const _Float16 *scale, const _Float16 *bias, int tile_col, int n, int m,
+                                                          int splits, int waves) {
     SkinnyScale s;
     const int tid = threadIdx.x;
-    if (m <= 4) {
+    if (skinny_column_layout(m, splits, waves)) {
         const int col = tile_col + (tid & 255);
         if (col < n) {
             s.one = scale[col];
@@ -294,7 +306,7 @@ __device__ __forceinline__ void skinny_finish(const float4_t (&res)[16], int m, 
     }
     __syncthreads();
 
-    if (m <= 4) {
+    if (skinny_column_layout(m, splits, WAVES)) {
         SkinnyTail<OutT, WAVES, 1> tail;
         tail.m = m;
         tail.n = n;

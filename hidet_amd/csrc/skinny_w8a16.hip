@@ -57,7 +57,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_kernel(const _Float16
 
     // the column factors this thread applies at the very end: fetched now, not looked at before then (a use here would
     // wait for the load before the first weight load is issued)
-    const SkinnyScale col_scale = skinny_fetch_scale(scale, bias, tile_col, n, m);
+    const SkinnyScale col_scale = skinny_fetch_scale(scale, bias, tile_col, n, m, splits, WAVES);
 
     float4_t acc[16];
 #pragma unroll
