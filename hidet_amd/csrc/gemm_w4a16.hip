@@ -618,13 +618,16 @@ __global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
     };
 
     // Dequantisation: thread (lane, wave) widens bytes `lane` (columns 2 lane, 2 lane + 1) of rows 8 wave .. 8 wave + 7.
-    const uint32_t raw_rd = uint32_t(Cfg::kRawBase + wave * 512 + lane);
+    // (the upper half of a wave takes the neighbouring k-group, wave ^ 1: a wave's two 16-byte writes of a stage then land on
+    // all sixteen 16-byte bank groups, four lanes each, instead of eight lanes on eight of them)
+    const int kgrp = wave ^ (lane >> 5);
+    const uint32_t raw_rd = uint32_t(Cfg::kRawBase + kgrp * 512 + lane);
     const uint32_t sc_rd = uint32_t(Cfg::kRawBase + 4096 + lane * 4);
     uint32_t bw_addr[2];
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
         const int sig = (lane >> 5) * 64 + (2 * (lane & 1) + e) * 16 + ((lane & 31) >> 1);
-        bw_addr[e] = uint32_t(Cfg::kBBase + (sig * 8 + (wave ^ lds_swizzle_key_step1(sig))) * 16);
+        bw_addr[e] = uint32_t(Cfg::kBBase + (sig * 8 + (kgrp ^ lds_swizzle_key_step1(sig))) * 16);
     }
     uint32_t bytes[8], sc2;
     auto read_raw = [&](int slot) {
