@@ -18,147 +18,160 @@ namespace {
 
 constexpr int kSkinnyWaves = 8;   // waves per workgroup; they split the workgroup's K slice
 constexpr int kNonTemporal = 2;   // cache policy bits of a buffer load: sc0 = 1, nt = 2, sc1 = 16
+#ifndef QMM_W4_FLAT
+#define QMM_W4_FLAT true
+#endif
 constexpr int kDepth = 2;          // 32-row steps fetched together
 
-// Same launch shape and load discipline as the int8 kernel: 8-wave workgroups in one round over the chip, one 32-row
-// step (8 loads of 8 bytes per lane, non-temporal) in flight per wave, no condition around a load - rows past the wave's
-// range lie outside the buffer and read as zero bytes, which are code 0 - and the split-K exchange of skinny_finish.
+// Same launch plan and load discipline as the int8 kernel: the (tile, 32-row step) units dealt evenly to 8-wave
+// workgroups, non-temporal loads with no condition around them - rows past the wave's range lie outside the buffer and
+// read as zero bytes, which are code 0 - and the exchange of skinny_tails. A step is 32 rows and the group size a
+// multiple of 32, so a step never straddles two groups.
 template <int DT, bool ALIGNED_A>
-__global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,
-                                                                        const uint8_t *__restrict__ w,
-                                                                        const uint16_t *__restrict__ scales,
-                                                                        uint16_t *__restrict__ c, int m, int k, int n, int group,
-                                                                        int rows_per_block, int splits, int tiles,
-                                                                        float *__restrict__ mailbox) {
+__global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(int ksteps, uint32_t ksteps_magic, int per_group, int longer, int splits, uint32_t splits_magic,
+                                                                        const uint8_t *__restrict__ w, const uint16_t *__restrict__ a,
+                                                                        int64_t lda, int m, int k, int n, int group,
+                                                                        SkinnyPlanRest plan_rest, const uint16_t *__restrict__ scales,
+                                                                        uint16_t *__restrict__ c, float *__restrict__ mailbox,
+                                                                        uint32_t *__restrict__ lost_flag) {
     using T = W4Traits<DT>;
     extern __shared__ float red[];
 
-    int tile, split;
-    if (!skinny_tile_of_block(splits, tiles, &tile, &split)) return;
+    const SkinnyPlanHead plan_head = {ksteps, ksteps_magic, per_group, longer, splits, splits_magic};
+    const SkinnyPlan plan(plan_head, plan_rest);
+    int grp;
+    if (!skinny_group_of_block(plan_head, plan_rest.tiles, int(blockIdx.x), &grp)) return;
+    const SkinnyWork wk = skinny_work_of(plan_head, grp);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, cl = lane & 15;
-    const int tile_col = tile * kSkinnyTileN;
-    const bool col_ok = tile_col + cl * 16 < n;
     const int row_bytes = n >> 1;
+    int run_lo, run_hi, part;
+    skinny_wave_run(wk, wave, kSkinnyWaves, &run_lo, &run_hi, &part);
 
-    const int rows_per_wave = rows_per_block / kSkinnyWaves;
-    const int k_begin = split * rows_per_block + wave * rows_per_wave;
-    const int k_end = min(k, k_begin + rows_per_wave);
-    const int nsteps = k_end > k_begin ? (k_end - k_begin + 31) >> 5 : 0;
-
-    float4_t acc[16], total[16];
-#pragma unroll
-    for (int t = 0; t < 16; ++t) {
-        acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-        total[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-    }
-    float4_t xsum = {0.f, 0.f, 0.f, 0.f};
     const uint32_t one2 = uint32_t(T::kOne) | (uint32_t(T::kOne) << 16);
     const uint4 ones = uint4{one2, one2, one2, one2};
-
-    // weights: the wave's rows at the tile's first byte column; a lane whose 16 columns lie past N reads the tile's
-    // first columns and its results are never stored
-    const int64_t w_bytes = int64_t(k_end - k_begin) * row_bytes - (tile_col >> 1);
-    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t *>(w + int64_t(k_begin) * row_bytes + (tile_col >> 1)), 0, int(w_bytes < 0 ? 0 : w_bytes), 0x00020000);
-    uint32_t w_off = uint32_t(8 * g) * uint32_t(row_bytes) + (col_ok ? cl * 8 : 0);
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(a), 0, ALIGNED_A ? int((int64_t(m - 1) * lda + k) * 2) : 0, 0x00020000);
     const uint16_t *ap = a + int64_t(cl) * lda;
     const int a_row_off = int(int64_t(cl) * lda * 2);
-    // scales of this lane's 16 columns: 32 bytes per group
+    // scales of a lane's 16 columns: 32 bytes per group
     const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(scales), 0, int(int64_t(k / group) * n * 2), 0x00020000);
-    const int s_col_off = (tile_col + (col_ok ? cl * 16 : 0)) * 2;
-    uint4v_t sc_raw[2] = {uint4v_t{0u, 0u, 0u, 0u}, uint4v_t{0u, 0u, 0u, 0u}};
 
-    // kDepth 32-row steps are fetched together: a step is only 4 KiB per wave here (8 bytes per lane and row). Measured at
-    // 4096 x 11008, one row: 1 / 2 / 4 steps 9.5 / 9.3 / 9.9 us; without any of the arithmetic below 8.3 - 8.6 us: the
-    // kernel's time is launch ramp, memory latency and the exchange, not the 23 MB it reads.
-    for (int step0 = 0; step0 < nsteps; step0 += kDepth) {
-        uint2 raw[kDepth][8];
-        uint4 xa[kDepth];
+    // the wave's run lies in one tile (skinny_wave_run)
+    {
+        const int tile = wk.tile + part;
+        const int tile_col = tile * kSkinnyTileN;
+        const bool col_ok = tile_col + cl * 16 < n;
+        const int k_begin = (run_lo - tile * plan.ksteps) * 32;
+        const int k_end = min(k, (run_hi - tile * plan.ksteps) * 32);
+        const int nsteps = run_hi - run_lo;
+
+        float4_t acc[16], total[16];
 #pragma unroll
-        for (int d = 0; d < kDepth; ++d) {
-#pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_off + uint32_t(r) * uint32_t(row_bytes), 0, kNonTemporal);
-                raw[d][r] = uint2{v[0], v[1]};
-            }
-            w_off += 32u * uint32_t(row_bytes);
-            asm volatile("" : "+v"(w_off));
-            const int kx = k_begin + 32 * (step0 + d) + 8 * g;
-            if (ALIGNED_A) {
-                const int off = (cl < m && kx < k_end) ? a_row_off + kx * 2 : 0x7FFFFFF0;
-                xa[d] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0));
-            } else {
-                uint16_t tmp[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) tmp[j] = (cl < m && kx + j < k_end) ? ap[kx + j] : uint16_t(0);
-                xa[d] = uint4{uint32_t(tmp[0]) | (uint32_t(tmp[1]) << 16), uint32_t(tmp[2]) | (uint32_t(tmp[3]) << 16),
-                              uint32_t(tmp[4]) | (uint32_t(tmp[5]) << 16), uint32_t(tmp[6]) | (uint32_t(tmp[7]) << 16)};
-            }
+        for (int t = 0; t < 16; ++t) {
+            acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+            total[t] = float4_t{0.f, 0.f, 0.f, 0.f};
         }
+        float4_t xsum = {0.f, 0.f, 0.f, 0.f};
+
+        // weights: the wave's rows at the tile's first byte column; a lane whose 16 columns lie past N reads the tile's
+        // first columns and its results are never stored
+        const int64_t w_bytes = int64_t(k_end - k_begin) * row_bytes - (tile_col >> 1);
+        const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t *>(w + int64_t(k_begin) * row_bytes + (tile_col >> 1)), 0, int(w_bytes < 0 ? 0 : w_bytes), 0x00020000);
+        uint32_t w_off = uint32_t(8 * g) * uint32_t(row_bytes) + (col_ok ? cl * 8 : 0);
+        const int s_col_off = (tile_col + (col_ok ? cl * 16 : 0)) * 2;
+        uint4v_t sc_raw[2] = {uint4v_t{0u, 0u, 0u, 0u}, uint4v_t{0u, 0u, 0u, 0u}};
+
+        // kDepth 32-row steps are fetched together: a step is only 4 KiB per wave here (8 bytes per lane and row).
+        for (int step0 = 0; step0 < nsteps; step0 += kDepth) {
+            uint2 raw[kDepth][8];
+            uint4 xa[kDepth];
 #pragma unroll
-        for (int d = 0; d < kDepth; ++d) {
-            const int step = step0 + d;
-            if (step >= nsteps) break;  // uniform across the wave
-            const int ks = k_begin + 32 * step;
-            if (ks % group == 0 || step == 0) {  // a new group starts
-                const int soff = (ks / group) * n * 2 + s_col_off;
-                sc_raw[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, soff, 0, 0);
-                sc_raw[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, soff + 16, 0, 0);
-            }
-            // byte b of dword h of rows 2p and 2p+1 goes to bits 0-7 and 16-23 of one register (v_perm_b32); its low
-            // nibbles are column 8h + 2b of both rows, its high nibbles column 8h + 2b + 1: mask-and-xor (one
-            // three-input bit operation) gives the two 16-bit floats bias + q, for the odd column after a shift
+            for (int d = 0; d < kDepth; ++d) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+                for (int r = 0; r < 8; ++r) {
+                    const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_off + uint32_t(r) * uint32_t(row_bytes), 0, kNonTemporal);
+                    raw[d][r] = uint2{v[0], v[1]};
+                }
+                w_off += 32u * uint32_t(row_bytes);
+                asm volatile("" : "+v"(w_off));
+                const int kx = k_begin + 32 * (step0 + d) + 8 * g;
+                if (ALIGNED_A) {
+                    const int off = (cl < m && kx < k_end) ? a_row_off + kx * 2 : 0x7FFFFFF0;
+                    xa[d] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0));
+                } else {
+                    uint16_t tmp[8];
 #pragma unroll
-                for (int byte = 0; byte < 4; ++byte) {
-                    constexpr uint32_t kZero = 0x0c;
-                    const uint32_t sel = (kZero << 24) | (uint32_t(4 + byte) << 16) | (kZero << 8) | uint32_t(byte);
-                    uint4 be, bo;
-                    uint32_t *bep = reinterpret_cast<uint32_t *>(&be), *bop = reinterpret_cast<uint32_t *>(&bo);
-#pragma unroll
-                    for (int p = 0; p < 4; ++p) {
-                        const uint32_t lo = h ? raw[d][2 * p].y : raw[d][2 * p].x;
-                        const uint32_t hi = h ? raw[d][2 * p + 1].y : raw[d][2 * p + 1].x;
-                        const uint32_t x = __builtin_amdgcn_perm(hi, lo, sel);
-                        bep[p] = (x & 0x000F000Fu) ^ T::kMagic;
-                        bop[p] = ((x >> 4) & 0x000F000Fu) ^ T::kMagic;
-                    }
-                    const int t = 8 * h + 2 * byte;
-                    acc[t] = T::mfma(xa[d], be, acc[t]);
-                    acc[t + 1] = T::mfma(xa[d], bo, acc[t + 1]);
+                    for (int j = 0; j < 8; ++j) tmp[j] = (cl < m && kx + j < k_end) ? ap[kx + j] : uint16_t(0);
+                    xa[d] = uint4{uint32_t(tmp[0]) | (uint32_t(tmp[1]) << 16), uint32_t(tmp[2]) | (uint32_t(tmp[3]) << 16),
+                                  uint32_t(tmp[4]) | (uint32_t(tmp[5]) << 16), uint32_t(tmp[6]) | (uint32_t(tmp[7]) << 16)};
                 }
             }
-            xsum = T::mfma(xa[d], ones, xsum);
-            if ((ks + 32) % group == 0 || step == nsteps - 1) {  // group complete (or the wave's range ends): fold it in
-                const uint16_t *sv = reinterpret_cast<const uint16_t *>(sc_raw);
 #pragma unroll
-                for (int t = 0; t < 16; ++t) {
-                    const float s = T::to_f32(sv[t]);
-                    const float sb = -T::kBias * s;  // exact: a power of two plus a small multiple times a 16-bit float
+            for (int d = 0; d < kDepth; ++d) {
+                const int step = step0 + d;
+                if (step >= nsteps) break;  // uniform across the wave
+                const int ks = k_begin + 32 * step;
+                if (ks % group == 0 || step == 0) {  // a new group starts
+                    const int soff = (ks / group) * n * 2 + s_col_off;
+                    sc_raw[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, soff, 0, 0);
+                    sc_raw[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_s, soff + 16, 0, 0);
+                }
+                // byte b of dword h of rows 2p and 2p+1 goes to bits 0-7 and 16-23 of one register (v_perm_b32); its low
+                // nibbles are column 8h + 2b of both rows, its high nibbles column 8h + 2b + 1: mask-and-xor (one
+                // three-input bit operation) gives the two 16-bit floats bias + q, for the odd column after a shift
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        total[t][v] = fmaf(acc[t][v], s, total[t][v]);
-                        total[t][v] = fmaf(xsum[v], sb, total[t][v]);
-                        acc[t][v] = 0.f;
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int byte = 0; byte < 4; ++byte) {
+                        constexpr uint32_t kZero = 0x0c;
+                        const uint32_t sel = (kZero << 24) | (uint32_t(4 + byte) << 16) | (kZero << 8) | uint32_t(byte);
+                        uint4 be, bo;
+                        uint32_t *bep = reinterpret_cast<uint32_t *>(&be), *bop = reinterpret_cast<uint32_t *>(&bo);
+#pragma unroll
+                        for (int p = 0; p < 4; ++p) {
+                            const uint32_t lo32 = h ? raw[d][2 * p].y : raw[d][2 * p].x;
+                            const uint32_t hi32 = h ? raw[d][2 * p + 1].y : raw[d][2 * p + 1].x;
+                            const uint32_t x = __builtin_amdgcn_perm(hi32, lo32, sel);
+                            bep[p] = (x & 0x000F000Fu) ^ T::kMagic;
+                            bop[p] = ((x >> 4) & 0x000F000Fu) ^ T::kMagic;
+                        }
+                        const int t = 8 * h + 2 * byte;
+                        acc[t] = T::mfma(xa[d], be, acc[t]);
+                        acc[t + 1] = T::mfma(xa[d], bo, acc[t + 1]);
                     }
                 }
-                xsum = float4_t{0.f, 0.f, 0.f, 0.f};
+                xsum = T::mfma(xa[d], ones, xsum);
+                if ((ks + 32) % group == 0 || step == nsteps - 1) {  // group complete (or the wave's range ends): fold it in
+                    const uint16_t *sv = reinterpret_cast<const uint16_t *>(sc_raw);
+#pragma unroll
+                    for (int t = 0; t < 16; ++t) {
+                        const float s = T::to_f32(sv[t]);
+                        const float sb = -T::kBias * s;  // exact: a power of two plus a small multiple times a 16-bit float
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            total[t][v] = fmaf(acc[t][v], s, total[t][v]);
+                            total[t][v] = fmaf(xsum[v], sb, total[t][v]);
+                            acc[t][v] = 0.f;
+                        }
+                    }
+                    xsum = float4_t{0.f, 0.f, 0.f, 0.f};
+                }
             }
         }
+        skinny_stash(total, m, wave, red);
     }
     const SkinnyScale no_scale;  // ones and no bias: the group scales are already in the totals
+    const SkinnyRoles roles = skinny_roles_of(plan, wk, grp, kSkinnyWaves);
     if (DT == HIDET_QMM_F16)
-        skinny_finish<_Float16, kSkinnyWaves>(total, m, n, tile, split, splits, no_scale, reinterpret_cast<_Float16 *>(c), mailbox, red);
+        skinny_tails<_Float16, kSkinnyWaves>(plan, wk, roles, m, n, no_scale, reinterpret_cast<_Float16 *>(c), mailbox, lost_flag, red);
     else
-        skinny_finish<uint16_t, kSkinnyWaves>(total, m, n, tile, split, splits, no_scale, c, mailbox, red);
+        skinny_tails<uint16_t, kSkinnyWaves>(plan, wk, roles, m, n, no_scale, c, mailbox, lost_flag, red);
 }
 
 // Any shape the fast kernel cannot take: one thread per output element, serial K, fp32 accumulation.
@@ -187,7 +200,7 @@ __global__ __launch_bounds__(256) void naive_w4a16_kernel(const uint16_t *__rest
 }  // namespace
 
 bool skinny_w4a16_fast(const void *w, const void *scales, int64_t k, int64_t n, int group) {
-    return (n % 16 == 0) && (group % 32 == 0) && aligned(w, 8) && aligned(scales, 16) && k > 0;
+    return (n % 16 == 0) && n < (int64_t(1) << 30) && (group % 32 == 0) && aligned(w, 8) && aligned(scales, 16) && k > 0;
 }
 
 void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
@@ -204,12 +217,11 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
             launch(naive_w4a16_kernel<HIDET_QMM_BF16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
         return;
     }
-    int rpb, splits, tiles;
-    skinny_plan_one_round(k, n, kSkinnyWaves, parallel_k_parts, &rpb, &splits, &tiles);
     const Workspace ws = split_workspace(workspace, workspace_bytes);
-    skinny_fit_mailbox(k, 32 * kSkinnyWaves, tiles, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, &rpb, &splits);
-    // a wave's K range and the scale table are addressed with 31-bit offsets
-    if ((int64_t(rpb) / kSkinnyWaves + 64) * (n / 2) >= (int64_t(1) << 31) - (1 << 20) || (k / group) * n * 2 >= (int64_t(1) << 31) - (1 << 20)) {
+    const SkinnyPlan plan = skinny_make_plan(k, n, parallel_k_parts, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, QMM_W4_FLAT);
+    // a wave's run of rows and the scale table are addressed with 31-bit offsets
+    if ((cdiv(cdiv(skinny_units(plan), plan.groups), kSkinnyWaves) * 32 + 64) * (n / 2) >= (int64_t(1) << 31) - (1 << 20) ||
+        (k / group) * n * 2 >= (int64_t(1) << 31) - (1 << 20)) {
         if (dtype == HIDET_QMM_F16)
             launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
         else
@@ -218,14 +230,15 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     }
     // 16-byte activation loads through a buffer descriptor: aligned rows, offsets below 2^31
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16) && (15 * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
-    const int grid = int(cdiv(tiles, 8) * 8 * splits);
+    uint32_t *lost_flag = ws.counters != nullptr ? ws.counters + kSkinnyLostWord : nullptr;
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
         const size_t shmem = skinny_lds_bytes(mt, kSkinnyWaves);
         auto go = [&](auto kern) {
             if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16, kSkinnyWaves)));  // the most any m needs
-            launch(kern, dim3(grid), dim3(64 * kSkinnyWaves), shmem, stream, ap0 + m0 * lda, lda, wp, sp, cp0 + m0 * n, mt, int(k),
-                   int(n), group, rpb, splits, tiles, ws.mailbox);
+            launch(kern, dim3(skinny_grid(plan)), dim3(64 * kSkinnyWaves), shmem, stream, plan.ksteps, plan.ksteps_magic, plan.per_group, plan.longer, plan.splits, plan.splits_magic,
+                   wp, ap0 + m0 * lda, lda, mt, int(k), int(n), group, static_cast<SkinnyPlanRest>(plan), sp, cp0 + m0 * n, ws.mailbox,
+                   lost_flag);
         };
         if (dtype == HIDET_QMM_F16) {
             if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, true>);

@@ -1,5 +1,5 @@
 // Host-side enumeration of launches: every tile of the output must be computed exactly once (all of its K ranges or
-// slices, each by one workgroup), and GEMM tiles that are split must get distinct fix-up slots inside the planned storage.
+// steps, each by one workgroup or wave), and GEMM tiles that are split must get distinct fix-up slots inside the planned storage.
 // Built and run by tests/test_tiling.py; exits non-zero with a message on the first violation.
 #include <cstdio>
 #include <vector>
@@ -54,37 +54,11 @@ static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_par
     return 0;
 }
 
-// Bandwidth-bound kernels: K is cut into `splits` slices of rows_per_block rows (whole multiples of the granule) that
-// cover K exactly once, and every (column tile, slice) pair belongs to exactly one workgroup.
-static int check_skinny(long long k, long long ncols, int slice_rows, int hint, int granule) {
-    int rpb = 0, splits = 0, tiles = 0;
-    if (slice_rows > 0) skinny_plan(k, ncols, slice_rows, hint, granule, &rpb, &splits, &tiles);
-    else skinny_plan_one_round(k, ncols, granule / 32, hint, &rpb, &splits, &tiles);  // the int8 kernel's plan
-    if (slice_rows == 0 && hint == 0 && (long long)(splits) * tiles > 256 && splits > 1)
-        return std::printf("skinny k=%lld n=%lld: %d slices x %d tiles do not fit one round\n", k, ncols, splits, tiles), 1;
-    if (rpb <= 0 || rpb % granule != 0 || splits < 1 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
-        tiles != int((ncols + kSkinnyTileN - 1) / kSkinnyTileN))
-        return std::printf("skinny k=%lld n=%lld hint=%d: rows %d x %d splits, %d tiles\n", k, ncols, hint, rpb, splits, tiles), 1;
-    std::vector<int> seen(size_t(tiles) * splits, 0);
-    const int grid = ((tiles + 7) / 8) * 8 * splits;
-    for (int b = 0; b < grid; ++b) {
-        int tile, split;
-        if (!skinny_tile_of(b, splits, tiles, &tile, &split)) continue;
-        if (tile < 0 || split < 0 || split >= splits || seen[size_t(tile) * splits + split]++)
-            return std::printf("skinny k=%lld n=%lld: block %d -> tile %d split %d\n", k, ncols, b, tile, split), 1;
-    }
-    for (int v : seen)
-        if (v != 1) return std::printf("skinny k=%lld n=%lld: a slice has no workgroup\n", k, ncols), 1;
-    return 0;
-}
-
-// A plan cut down to a mailbox: still whole granules covering K once, never more bytes than the mailbox holds, the
-// plan untouched when it fits, and a strict caller gets an error exactly when it does not.
-static int check_fit(long long k, long long ncols, int rows, long long workspace_bytes, int granule) {
-    int rpb = 0, splits = 0, tiles = 0;
-    if (granule == 256) skinny_plan_one_round(k, ncols, 8, 0, &rpb, &splits, &tiles);
-    else skinny_plan(k, ncols, rows > 8 ? 768 : 512, 0, granule, &rpb, &splits, &tiles);
-    const int rpb0 = rpb, splits0 = splits;
+// Bandwidth-bound kernels: the (tile, 32-row step) units of a launch are dealt to workgroups and waves in one flat run
+// each. Every unit must belong to exactly one wave, a workgroup's run may touch two tiles at most, every tile has one
+// collector (the workgroup with its last unit) that fetches exactly the slots of the workgroups before it in the tile,
+// every other contributor sends exactly once into its own slot, and the plan never needs more mailbox than there is.
+static int check_skinny(long long k, long long ncols, int hint, int rows, long long workspace_bytes) {
     static char dummy[16];
     const Workspace ws = split_workspace(dummy, workspace_bytes);
     if (workspace_bytes >= kCounterBytes &&
@@ -92,40 +66,115 @@ static int check_fit(long long k, long long ncols, int rows, long long workspace
          kCounterBytes + ws.mailbox_bytes + ws.scratch_bytes != workspace_bytes ||
          reinterpret_cast<char *>(ws.mailbox) + ws.mailbox_bytes != ws.scratch))
         return std::printf("workspace of %lld bytes: mailbox %lld, scratch %lld\n", workspace_bytes, (long long)ws.mailbox_bytes, (long long)ws.scratch_bytes), 1;
-    const bool fits = skinny_mailbox_need(tiles, splits, rows) <= ws.mailbox_bytes;
+    const SkinnyPlan free_plan = skinny_make_plan(k, ncols, hint, rows, 1LL << 40, true);
+    const bool fits = skinny_mailbox_need(free_plan, rows) <= ws.mailbox_bytes;
     bool threw = false;
     try {
-        int r2 = rpb, s2 = splits;
-        skinny_fit_mailbox(k, granule, tiles, rows, ws.mailbox_bytes, true, &r2, &s2);
+        skinny_make_plan(k, ncols, hint, rows, ws.mailbox_bytes, true);
     } catch (const Error &) { threw = true; }
-    if (threw == fits) return std::printf("fit k=%lld n=%lld rows=%d ws=%lld: strict error %d, fits %d\n", k, ncols, rows, workspace_bytes, threw, fits), 1;
-    skinny_fit_mailbox(k, granule, tiles, rows, ws.mailbox_bytes, false, &rpb, &splits);
-    if (fits && (rpb != rpb0 || splits != splits0)) return std::printf("fit k=%lld n=%lld: a plan that fits was changed\n", k, ncols), 1;
-    if (rpb <= 0 || rpb % granule != 0 || splits < 1 || splits > splits0 || (long long)(splits) * rpb < k || (long long)(splits - 1) * rpb >= k ||
-        skinny_mailbox_need(tiles, splits, rows) > ws.mailbox_bytes)
-        return std::printf("fit k=%lld n=%lld rows=%d ws=%lld: rows %d x %d splits need %lld\n", k, ncols, rows, workspace_bytes, rpb, splits,
-                           (long long)skinny_mailbox_need(tiles, splits, rows)), 1;
+    if (threw == fits) return std::printf("skinny k=%lld n=%lld rows=%d ws=%lld: strict error %d, fits %d\n", k, ncols, rows, workspace_bytes, threw, fits), 1;
+    const SkinnyPlan p = skinny_make_plan(k, ncols, hint, rows, ws.mailbox_bytes, false);
+    if (fits && (p.groups != free_plan.groups)) return std::printf("skinny k=%lld n=%lld: a plan that fits was changed\n", k, ncols), 1;
+    const int units = skinny_units(p);
+    if (p.tiles != int((ncols + kSkinnyTileN - 1) / kSkinnyTileN) || p.ksteps != int((k + 31) / 32) || p.groups < p.tiles ||
+        p.groups > units || p.groups > free_plan.groups || skinny_mailbox_need(p, rows) > ws.mailbox_bytes)
+        return std::printf("skinny k=%lld n=%lld hint=%d rows=%d ws=%lld: %d tiles x %d steps, %d workgroups need %lld\n", k, ncols, hint, rows,
+                           workspace_bytes, p.tiles, p.ksteps, p.groups, (long long)skinny_mailbox_need(p, rows)), 1;
+    if (hint == 0 && p.groups > 256 && p.groups != p.tiles)
+        return std::printf("skinny k=%lld n=%lld: %d workgroups do not fit one round\n", k, ncols, p.groups), 1;
+    constexpr int kWaves = 8;
+    std::vector<int> seen(units, 0), collector(p.tiles, -1), first(p.tiles, -1), sends(p.groups, 0), sent_to(p.groups, -1);
+    int most = 0;
+    // every run belongs to exactly one workgroup of the launch; with whole runs per tile a tile's runs share an XCD
+    // (workgroup index mod 8) and are dispatched in run order
+    std::vector<int> block_of(p.groups, -1);
+    for (int b = 0; b < skinny_grid(p); ++b) {
+        int g = -1;
+        if (!skinny_group_of_block(p, p.tiles, b, &g)) continue;
+        if (g < 0 || g >= p.groups || block_of[g] >= 0) return std::printf("skinny k=%lld n=%lld: workgroup %d -> run %d\n", k, ncols, b, g), 1;
+        block_of[g] = b;
+    }
+    for (int g = 0; g < p.groups; ++g) {
+        if (block_of[g] < 0) return std::printf("skinny k=%lld n=%lld: run %d has no workgroup\n", k, ncols, g), 1;
+        if (p.splits > 0 && g % p.splits != 0 && (block_of[g] % 8 != block_of[g - 1] % 8 || block_of[g] < block_of[g - 1]))
+            return std::printf("skinny k=%lld n=%lld: runs %d and %d of one tile on workgroups %d and %d\n", k, ncols, g - 1, g, block_of[g - 1], block_of[g]), 1;
+    }
+    if (p.splits > 0 && p.groups != p.tiles * p.splits) return std::printf("skinny k=%lld n=%lld: %d splits, %d runs, %d tiles\n", k, ncols, p.splits, p.groups, p.tiles), 1;
+    for (int g = 0; g < p.groups; ++g) {
+        const SkinnyWork wk = skinny_work_of(p, g);
+        if (p.splits > 0 && (wk.crosses() || wk.tile != g / p.splits)) return std::printf("skinny k=%lld n=%lld: run %d of %d per tile crosses out of tile %d\n", k, ncols, g, p.splits, wk.tile), 1;
+        if (wk.u0 != skinny_first_unit(p, g) || wk.u1 <= wk.u0 || wk.u1 > units || wk.tile != wk.u0 / p.ksteps ||
+            (wk.u1 - 1) / p.ksteps > wk.tile + 1 || skinny_group_of_unit(p, wk.u0) != g || skinny_group_of_unit(p, wk.u1 - 1) != g)
+            return std::printf("skinny k=%lld n=%lld: workgroup %d runs [%d, %d) from tile %d\n", k, ncols, g, wk.u0, wk.u1, wk.tile), 1;
+        const SkinnyRoles roles = skinny_roles_of(p, wk, g, kWaves);
+        int at = wk.u0;
+        for (int wv = 0; wv < kWaves; ++wv) {
+            int lo, hi, part;
+            skinny_wave_run(wk, wv, kWaves, &lo, &hi, &part);
+            if (lo != at || hi < lo) return std::printf("skinny k=%lld n=%lld: workgroup %d wave %d runs [%d, %d), expected from %d\n", k, ncols, g, wv, lo, hi, at), 1;
+            // a wave's run lies in one tile, and its LDS slot (= its index) is one of that tile's
+            if (part != (wv >= roles.c0) || (part == 0 && hi > wk.bound) || (part == 1 && (lo < wk.bound || !wk.crosses())))
+                return std::printf("skinny k=%lld n=%lld: workgroup %d wave %d runs [%d, %d) for part %d, boundary at %d, %d waves before it\n", k, ncols, g, wv, lo, hi, part, wk.bound, roles.c0), 1;
+            if (hi - lo > (wk.u1 - wk.u0 + kWaves - 2) / (kWaves - 1) + 1)  // two groups of waves: no wave beyond a seventh of the run (and rounding)
+                return std::printf("skinny k=%lld n=%lld: workgroup %d wave %d has %d of %d steps\n", k, ncols, g, wv, hi - lo, wk.u1 - wk.u0), 1;
+            for (int u = lo; u < hi; ++u) ++seen[u];
+            at = hi;
+        }
+        if (at != wk.u1) return std::printf("skinny k=%lld n=%lld: workgroup %d waves end at %d, run at %d\n", k, ncols, g, at, wk.u1), 1;
+        if (roles.c0 < 1 || roles.c0 > kWaves || (wk.crosses() && roles.c0 == kWaves))
+            return std::printf("skinny k=%lld n=%lld: workgroup %d: %d waves before the boundary\n", k, ncols, g, roles.c0), 1;
+        // roles
+        if (first[wk.tile] < 0) first[wk.tile] = g;
+        if (roles.finish != int(wk.collects()) || (roles.send_slot >= 0) != (wk.crosses() || !wk.collects()) || (roles.send_slot >= 0 && roles.send_slot != g) ||
+            roles.send_tile != (wk.crosses() ? wk.tile + 1 : wk.tile) ||
+            (roles.send_slot >= 0 && (roles.send_lo != (wk.crosses() ? roles.c0 : 0) || roles.send_hi != kWaves)))
+            return std::printf("skinny k=%lld n=%lld: workgroup %d: finish %d, sends LDS slots [%d, %d) to slot %d for tile %d\n", k, ncols, g, roles.finish, roles.send_lo, roles.send_hi,
+                               roles.send_slot, roles.send_tile), 1;
+        if (wk.collects()) {
+            if (collector[wk.tile] >= 0) return std::printf("skinny k=%lld n=%lld: tile %d has two collectors\n", k, ncols, wk.tile), 1;
+            collector[wk.tile] = g;
+            if (roles.fetch_first != first[wk.tile] || roles.fetch_others != g - first[wk.tile])
+                return std::printf("skinny k=%lld n=%lld: workgroup %d fetches %d slots from %d, the tile's first is %d\n", k, ncols, g, roles.fetch_others, roles.fetch_first, first[wk.tile]), 1;
+            most = std::max(most, roles.fetch_others);
+        } else {
+            ++sends[g];
+            sent_to[g] = wk.tile;
+        }
+        if (wk.crosses()) {
+            if (wk.tile + 1 >= p.tiles || first[wk.tile + 1] >= 0) return std::printf("skinny k=%lld n=%lld: workgroup %d crosses into a tile that has begun\n", k, ncols, g), 1;
+            first[wk.tile + 1] = g;
+            ++sends[g];
+            sent_to[g] = wk.tile + 1;
+        } else if (wk.collects() && wk.tile + 1 < p.tiles && skinny_first_unit(p, g + 1) != wk.bound) {
+            return std::printf("skinny k=%lld n=%lld: workgroup %d ends at a tile boundary that the next does not start at\n", k, ncols, g), 1;
+        }
+    }
+    for (int u = 0; u < units; ++u)
+        if (seen[u] != 1) return std::printf("skinny k=%lld n=%lld: unit %d belongs to %d waves\n", k, ncols, u, seen[u]), 1;
+    for (int t = 0; t < p.tiles; ++t) {
+        if (collector[t] < 0 || first[t] < 0 || first[t] > collector[t]) return std::printf("skinny k=%lld n=%lld: tile %d has no collector\n", k, ncols, t), 1;
+        for (int g = first[t]; g < collector[t]; ++g)
+            if (sends[g] != 1 || sent_to[g] != t) return std::printf("skinny k=%lld n=%lld: workgroup %d should send once to tile %d\n", k, ncols, g, t), 1;
+    }
+    for (int g = 0; g < p.groups; ++g)
+        if (sends[g] > 1) return std::printf("skinny k=%lld n=%lld: workgroup %d sends twice\n", k, ncols, g), 1;
+    if (most != p.max_others) return std::printf("skinny k=%lld n=%lld: max_others %d, enumerated %d\n", k, ncols, p.max_others, most), 1;
+    if ((p.groups == p.tiles) != (most == 0)) return std::printf("skinny k=%lld n=%lld: %d workgroups, %d tiles, %d partial tiles fetched\n", k, ncols, p.groups, p.tiles, most), 1;
     return 0;
 }
 
 int main() {
     long long n = 0;
-    // 16384 x 128256 with 8 rows (an lm_head decode batch) wants 131 MB of partial tiles: it must come out within the mailbox
+    // 16384 x 128256 with 8 rows (an lm_head decode batch) has 501 tiles: one workgroup each, nothing exchanged; small
+    // workspaces cut a plan down to what their mailbox holds
     for (long long ws : {0LL, 1024LL, 65536LL, 65536LL + 8192, 1LL << 20, 16LL << 20, (16LL << 20) + 65536, 64LL << 20, 96LL << 20})
-        for (long long k : {128LL, 4096LL, 11008LL, 16384LL})
-            for (long long nc : {256LL, 4096LL, 11008LL, 128256LL})
+        for (long long k : {32LL, 96LL, 128LL, 1000LL, 4096LL, 11008LL, 16384LL, 28672LL})
+            for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL, 128256LL})
                 for (int rows : {1, 8, 16})
-                    for (int granule : {128, 256, 512}) {
-                        if (check_fit(k, nc, rows, ws, granule)) return 1;
+                    for (int hint : {0, 1, 3, 8, 64}) {
+                        if (check_skinny(k, nc, hint, rows, ws)) return 1;
                         ++n;
                     }
-    for (long long k : {32LL, 96LL, 128LL, 1000LL, 4096LL, 11008LL, 8192LL, 28672LL})
-        for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL})
-            for (int hint : {0, 1, 3, 8, 64})
-                for (int cfg = 0; cfg < 5; ++cfg) {
-                    if (check_skinny(k, nc, cfg == 1 ? 768 : cfg >= 3 ? 0 : 512, hint, cfg == 2 || cfg == 3 ? 256 : 128)) return 1;
-                    ++n;
-                }
     const int cfgs[][3] = {{32, 32, 4}, {32, 32, 8}, {64, 64, 4}, {64, 32, 4}};  // concurrent, fill, max_parts of the launchers
     for (const auto &c : cfgs)
         for (int tm = 1; tm <= 70; tm += (tm < 20 ? 1 : 7))
