@@ -107,6 +107,49 @@ HIDET_API void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w,
 
 HIDET_API int64_t hidet_qmm_static_scratch_bytes(void) { return kStaticScratchBytes; }
 
+namespace {
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint4 *__restrict__ dst, int64_t count) {
+    for (int64_t i = int64_t(blockIdx.x) * 256 + threadIdx.x; i < count; i += int64_t(gridDim.x) * 256) dst[i] = uint4{0u, 0u, 0u, 0u};
+}
+}  // namespace
+
+HIDET_API int hidet_qmm_exchange_status(const void *workspace, int64_t workspace_bytes, void *stream_) {
+    try {
+        const void *base = workspace;
+        if (base == nullptr) {
+            base = static_scratch_of_current_device();
+            workspace_bytes = kStaticScratchBytes;
+        }
+        hipStream_t stream = static_cast<hipStream_t>(stream_);
+        uint32_t word = 0;
+        if (workspace_bytes >= kCounterBytes)  // else: no counter block, no exchange ever ran on it
+            QMM_HIP(hipMemcpyAsync(&word, static_cast<const uint32_t *>(base) + kExchangeLostWord, sizeof(word), hipMemcpyDeviceToHost, stream));
+        QMM_HIP(hipStreamSynchronize(stream));
+        return word != 0u ? 1 : 0;
+    } catch (const std::exception &e) {
+        hidet_set_last_error(e.what());
+    } catch (...) {
+        hidet_set_last_error("unknown error");
+    }
+    return -1;
+}
+
+HIDET_API void hidet_qmm_exchange_reset(void *workspace, int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    if (workspace == nullptr) {
+        workspace = static_scratch_of_current_device();
+        workspace_bytes = kStaticScratchBytes;
+    }
+    QMM_CHECK(aligned(workspace, 16), "the workspace must be 16-byte aligned");
+    const Workspace ws = split_workspace(workspace, workspace_bytes);
+    if (ws.counters == nullptr) return;
+    // a fill kernel, not a memset node: callers may capture this into a graph
+    const int64_t count = (kCounterBytes + ws.mailbox_bytes) / 16;
+    launch_aux(zero_fill_kernel, dim3(uint32_t(std::min<int64_t>(2048, cdiv(count, 256)))), dim3(256), 0, static_cast<hipStream_t>(stream_),
+               static_cast<uint4 *>(workspace), count);
+    QMM_ENTRY_END
+}
+
 HIDET_API void hidet_symmetric_quant_matmul_f16_i8_static(const void *a, const void *w, const void *scale, void *c, int64_t m,
                                                           int64_t k, int64_t n, int64_t lda, int parallel_k_parts,
                                                           void *stream_) {

@@ -1,0 +1,141 @@
+// Measurement and test hooks of libhidet_qmm.so (include/hidet_qmm_bench.h): events and the per-launch timing hook,
+// kernels that only read, and the host-side switch of the exchange's give-up limit. Nothing an operator call needs.
+#include "common.h"
+#include "../../include/hidet_qmm_bench.h"
+
+HIDET_API void *hidet_qmm_event_create(void) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+        hidet_set_last_error("hipEventCreate failed");
+        return nullptr;
+    }
+    return e;
+}
+
+HIDET_API void hidet_qmm_event_destroy(void *event) {
+    if (event) (void)hipEventDestroy(static_cast<hipEvent_t>(event));
+}
+
+HIDET_API void hidet_qmm_event_record(void *event, void *stream) {
+    QMM_ENTRY_BEGIN
+    QMM_HIP(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_qmm_event_synchronize(void *event) {
+    QMM_ENTRY_BEGIN
+    QMM_HIP(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    QMM_ENTRY_END
+}
+
+HIDET_API float hidet_qmm_event_elapsed_ms(void *start, void *stop) {
+    float ms = -1.0f;
+    hipError_t e = hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop));
+    if (e != hipSuccess) {
+        hidet_set_last_error(hipGetErrorString(e));
+        return -1.0f;
+    }
+    return ms;
+}
+
+HIDET_API void hidet_qmm_arm_timing(void *start_event, void *stop_event) {
+    qmm::TimingSlot &ts = qmm::timing_slot();
+    ts.start = static_cast<hipEvent_t>(start_event);
+    ts.stop = static_cast<hipEvent_t>(stop_event);
+}
+
+HIDET_API void hidet_qmm_set_exchange_spin_limit(int limit) {
+    qmm::exchange_spin_limit().store(limit < 0 ? qmm::kExchangeSpinLimit : limit, std::memory_order_relaxed);
+}
+
+// ---- what a kernel that only reads can get out of the memory system ------------------------------------------------
+namespace {
+constexpr int kProbeBlockBytes = 32768;  // 256 threads x 8 loads x 16 bytes, contiguous per workgroup
+constexpr int kNonTemporal = 2;          // cache policy bits of a buffer load: sc0 = 1, nt = 2, sc1 = 16
+
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict__ src, uint32_t *__restrict__ sink) {
+    const uint4 *p = src + int64_t(blockIdx.x) * (kProbeBlockBytes / 16) + threadIdx.x;
+    uint4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = p[j * 256];
+    uint32_t acc = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    if (acc == 0x9E3779B9u) sink[0] = acc;  // practically never true; keeps the loads alive
+}
+
+// The loads of the decode kernel over an int8 matrix w[k, n] and nothing else: the (256-column tile, row) space is cut
+// into `workgroups` x 8 equal runs, one per wave; a wave walks its run in steps of 32 rows, a lane fetching 16 bytes of
+// each of 8 rows per step (a wave instruction covers four 256-byte row segments n bytes apart), one step in flight.
+// `contiguous`: the same bytes per wave, but as one 1 KiB piece per wave instruction.
+__global__ __launch_bounds__(512) void pattern_probe_kernel(const char *__restrict__ w, int n, int k, int tiles, int contiguous,
+                                                           uint32_t *__restrict__ sink) {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lg = lane >> 4, cl = lane & 15;
+    const int64_t space = int64_t(tiles) * k, runs = int64_t(gridDim.x) * 8;
+    const int64_t me = int64_t(blockIdx.x) * 8 + wave;
+    int64_t f0 = me * space / runs;
+    const int64_t f1 = (me + 1) * space / runs;
+    uint32_t acc = 0;
+    if (contiguous) {
+        const int64_t b0 = f0 * 256, b1 = f1 * 256;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(w + b0), 0, int(b1 - b0), 0x00020000);
+        const int loads = int((b1 - b0 + 1023) / 1024);
+        uint32_t off = lane * 16;
+        for (int s = 0; s < loads; s += 8) {
+            qmm::uint4v_t v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, off + j * 1024, 0, kNonTemporal);
+            off += 8 * 1024;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc += v[j][0] ^ v[j][1] ^ v[j][2] ^ v[j][3];
+        }
+    } else {
+        while (f0 < f1) {
+            const int tile = int(f0 / k);
+            const int r0 = int(f0 - int64_t(tile) * k);
+            const int64_t fend = f1 < int64_t(tile + 1) * k ? f1 : int64_t(tile + 1) * k;
+            const int rows = int(fend - f0);
+            // rows of the run, from the tile's first column: what lies behind reads as zero without going to memory
+            const int64_t bytes = int64_t(rows) * n - tile * 256;
+            const __amdgpu_buffer_rsrc_t rs =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(w + int64_t(r0) * n + tile * 256), 0, int(bytes), 0x00020000);
+            uint32_t off = uint32_t(8 * lg) * uint32_t(n) + cl * 16;
+            const int steps = (rows + 31) >> 5;
+            for (int s = 0; s < steps; ++s) {
+                qmm::uint4v_t v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, off + uint32_t(j) * uint32_t(n), 0, kNonTemporal);
+                off += 32u * uint32_t(n);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc += v[j][0] ^ v[j][1] ^ v[j][2] ^ v[j][3];
+            }
+            f0 = fend;
+        }
+    }
+    if (acc == 0x9E3779B9u) sink[0] = acc;
+}
+}  // namespace
+
+HIDET_API void hidet_qmm_read_probe(const void *src, int64_t bytes, void *sink, void *stream) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(src && sink && qmm::aligned(src, 16), "null or misaligned pointer");
+    QMM_CHECK(bytes > 0 && bytes % kProbeBlockBytes == 0 && bytes / kProbeBlockBytes < (int64_t(1) << 31),
+              "the size must be a positive multiple of " << kProbeBlockBytes << " bytes, got " << bytes);
+    qmm::launch(read_probe_kernel, dim3(uint32_t(bytes / kProbeBlockBytes)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                static_cast<const uint4 *>(src), static_cast<uint32_t *>(sink));
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_qmm_pattern_probe(const void *w, int64_t k, int64_t n, int workgroups, int contiguous, void *sink,
+                                       void *stream) {
+    QMM_ENTRY_BEGIN
+    QMM_CHECK(w && sink && qmm::aligned(w, 16), "null or misaligned pointer");
+    QMM_CHECK(k > 0 && n > 0 && n % 256 == 0 && k % 32 == 0, "the probe takes K a multiple of 32 and N a multiple of 256, got " << k << " x " << n);
+    QMM_CHECK(workgroups > 0 && workgroups <= 65536, "workgroups must be in [1, 65536], got " << workgroups);
+    // a wave's run is addressed with 31-bit offsets
+    QMM_CHECK((k * (n / 256) / (int64_t(workgroups) * 8) + 64) * n < (int64_t(1) << 31), "too few workgroups for a matrix of " << k << " x " << n);
+    qmm::launch(pattern_probe_kernel, dim3(uint32_t(workgroups)), dim3(512), 0, static_cast<hipStream_t>(stream),
+                static_cast<const char *>(w), int(n), int(k), int(n / 256), contiguous, static_cast<uint32_t *>(sink));
+    QMM_ENTRY_END
+}

@@ -4,8 +4,10 @@
 #include <hip/hip_ext.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdint>
 #include <exception>
+#include <map>
 #include <mutex>
 #include <set>
 #include <sstream>
@@ -110,6 +112,21 @@ inline void allow_dynamic_lds(const void *kernel, int bytes) {
     done.insert({kernel, device});
 }
 
+// Compute units of the current device, read once per device.
+inline int device_cus() {
+    static std::mutex mu;
+    static std::map<int, int> known;
+    int device = 0;
+    QMM_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> guard(mu);
+    auto it = known.find(device);
+    if (it != known.end()) return it->second;
+    int cus = 0;
+    QMM_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    known[device] = cus;
+    return cus;
+}
+
 // Helper kernels (fills, conversions) never consume the timing slot.
 template <typename... KArgs, typename... Args>
 inline void launch_aux(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args) {
@@ -136,6 +153,16 @@ typedef unsigned int uint4v_t __attribute__((ext_vector_type(4)));
 // nobody relies on between launches.
 constexpr int64_t kCounterBytes = 64 << 10;
 constexpr int64_t kMaxMailboxBytes = 16 << 20;
+// Word of the counter block (in its last 256 bytes, far behind the arrival counters) that a collector of the split-K
+// exchange sets when it gives up waiting for a partial tile. It stays set until hidet_qmm_exchange_reset.
+constexpr int kExchangeLostWord = 16320;
+// Re-reads of the mailbox after which a collector gives up: about a second of polling. Tests lower it from the host to
+// drive the give-up path without a kernel that waits for long.
+constexpr int kExchangeSpinLimit = 1 << 20;
+inline std::atomic<int> &exchange_spin_limit() {
+    static std::atomic<int> limit{kExchangeSpinLimit};
+    return limit;
+}
 
 struct Workspace {
     uint32_t *counters = nullptr;

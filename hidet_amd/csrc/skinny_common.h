@@ -214,9 +214,7 @@ __host__ __device__ __forceinline__ SkinnyRoles skinny_roles_of(const SkinnyPlan
 // no word is zero, adds them in workgroup order (its own last: the result does not depend on timing), writes the output
 // and puts the zeros back with plain stores, which the end of the kernel makes visible to the next launch. The wait is
 // bounded: after SkinnyPlan::spin_limit re-reads the output is NaN instead of a hang, the slots are cleared all the
-// same and a word of the workspace's counter block records the loss (kSkinnyLostWord) for the host to find.
-constexpr int kSkinnySpinLimit = 1 << 20;
-constexpr int kSkinnyLostWord = 16320;  // index of the flag in the workspace's 64 KiB counter block (its last 256 bytes)
+// same and a word of the workspace's counter block records the loss (kExchangeLostWord) for the host to find.
 
 // Which of the tail's two thread layouts a launch uses: one column per thread (dwords, `waves / 4` rows at a time) while a
 // thread's reads of the exchange are few - rows per thread x partial tiles to fetch within 4 x 4, 2 x 8 or 1 x 16 - and
@@ -398,6 +396,8 @@ struct SkinnyTail {
         // a trip: one output row of this thread and up to 8 or 16 slots (two rows of 8 slots per trip were measured
         // slower than two trips: 16 rows at 4096 x 11008 16.3 against 14.2 us)
         if (roles.fetch_others > 8) collect<1, 16>(mailbox, roles, send_slot);
+        else if (roles.fetch_others <= 4 && m > 2 * kRowGroups) collect<4, 4>(mailbox, roles, send_slot);
+        else if (roles.fetch_others <= 4 && m > kRowGroups) collect<2, 4>(mailbox, roles, send_slot);
         else collect<1, 8>(mailbox, roles, send_slot);
     }
 
@@ -588,12 +588,13 @@ __device__ __forceinline__ void skinny_tails(const SkinnyPlan &plan, const Skinn
 
 // ---- host side: the plan of a launch ------------------------------------------------------------------------------
 
-constexpr int kSkinnyGroups = 256;           // one workgroup per CU of a full MI355X
-constexpr int kSkinnyMinUnitsPerGroup = 16;  // two 32-row steps per wave of an 8-wave workgroup
+constexpr int kSkinnyGroups = 256;           // most workgroups of a plan: one per CU of a full MI355X
+constexpr int kSkinnyPlanWaves = 8;          // waves of a workgroup of the kernels that use the plan
+constexpr int kSkinnyMinUnitsPerGroup = 2 * kSkinnyPlanWaves;  // two 32-row steps per wave
 // The runs ignore the tile boundaries up to this many activation rows and while a tile has no more than this many
 // contributors; beyond, whole runs per tile with a tile's runs on one XCD are faster (one row at 11008 x 4096, 16 tiles:
 // 12.4 against 10.4 us; 16 rows at 4096 x 4096: 12.0 against 10.4 us).
-constexpr int kSkinnyFlatRows = 8, kSkinnyFlatSharers = 8;
+constexpr int kSkinnyFlatRows = 2, kSkinnyFlatSharers = 8;
 
 // Bytes of mailbox a plan touches: one fp32 partial tile of `rows` (at most 16) activation rows per workgroup, slot =
 // workgroup index. A plan of one workgroup per tile exchanges nothing.
@@ -615,18 +616,28 @@ inline int skinny_max_others(const SkinnyPlan &p) {
 // `hint_parts` > 0 asks for that many workgroups per tile instead. The partial tiles must fit the mailbox: a plan that
 // does not is cut down to fewer workgroups (one per tile needs no mailbox at all); `strict` callers get an error
 // instead, naming the bytes the plan needs.
-inline SkinnyPlan skinny_make_plan(int64_t k, int64_t n, int hint_parts, int rows, int64_t mailbox_bytes, bool strict, bool flat_ok = true) {
+inline SkinnyPlan skinny_make_plan(int64_t k, int64_t n, int hint_parts, int rows, int64_t mailbox_bytes, bool strict, bool flat_ok = true,
+                                   int cus = kSkinnyGroups) {
     SkinnyPlan p;
     const int64_t tiles = cdiv(n, kSkinnyTileN), ksteps = cdiv(k, 32), units = tiles * ksteps;
     QMM_CHECK(units < (int64_t(1) << 30), "K x N too large for one launch of the bandwidth-bound kernel: " << k << " x " << n);
     p.tiles = int(tiles);
     p.ksteps = int(ksteps);
+    // one workgroup per CU of the device the launch goes to (fewer CUs than a full MI355X: a partition, a CU mask known to
+    // the runtime), never more than 256: the mailbox bound of the callers is stated for that many
+    const int64_t most = std::max(1, std::min(cus, kSkinnyGroups));
     // few rows: as many workgroups as there are CUs, whatever the number of tiles; many rows (or a number of parts asked
     // for): whole runs per tile, a tile's runs on one XCD
     int64_t splits = hint_parts > 0 ? std::min<int64_t>(hint_parts, ksteps) : 0;
-    if (splits == 0 && (!flat_ok || rows > kSkinnyFlatRows || tiles * kSkinnyFlatSharers < kSkinnyGroups))
-        splits = std::max<int64_t>(1, std::min<int64_t>(kSkinnyGroups / tiles, units / kSkinnyMinUnitsPerGroup / tiles));
-    int64_t groups = splits > 0 ? tiles * splits : std::max<int64_t>(tiles, std::min<int64_t>(kSkinnyGroups, units / kSkinnyMinUnitsPerGroup));
+    if (splits == 0 && (!flat_ok || rows > kSkinnyFlatRows || tiles * kSkinnyFlatSharers < most))
+    {
+        splits = std::max<int64_t>(1, std::min<int64_t>(most / tiles, units / kSkinnyMinUnitsPerGroup / tiles));
+        // a launch takes as long as its busiest wave: no more slices than that wave's number of steps needs (4096 rows: 4
+        // slices of 4 steps per wave, not 5 of 3 or 4)
+        const auto wave_steps = [&](int64_t sl) { return cdiv(cdiv(ksteps, sl), kSkinnyPlanWaves); };
+        while (splits > 1 && wave_steps(splits - 1) == wave_steps(splits)) --splits;
+    }
+    int64_t groups = splits > 0 ? tiles * splits : std::max<int64_t>(tiles, std::min<int64_t>(most, units / kSkinnyMinUnitsPerGroup));
     p.groups = int(groups);
     const int64_t slot_bytes = int64_t(rows) * kSkinnyTileN * 4;
     if (skinny_mailbox_need(p, rows) > mailbox_bytes) {
@@ -646,7 +657,7 @@ inline SkinnyPlan skinny_make_plan(int64_t k, int64_t n, int hint_parts, int row
     p.ksteps_magic = skinny_magic(uint32_t(p.ksteps));
     p.per_group_magic = skinny_magic(uint32_t(p.per_group));
     p.per_group1_magic = skinny_magic(uint32_t(p.per_group + 1));
-    p.spin_limit = kSkinnySpinLimit;
+    p.spin_limit = exchange_spin_limit().load(std::memory_order_relaxed);
     p.max_others = skinny_max_others(p);
     return p;
 }

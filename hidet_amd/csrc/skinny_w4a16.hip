@@ -18,9 +18,6 @@ namespace {
 
 constexpr int kSkinnyWaves = 8;   // waves per workgroup; they split the workgroup's K slice
 constexpr int kNonTemporal = 2;   // cache policy bits of a buffer load: sc0 = 1, nt = 2, sc1 = 16
-#ifndef QMM_W4_FLAT
-#define QMM_W4_FLAT true
-#endif
 constexpr int kDepth = 2;          // 32-row steps fetched together
 
 // Same launch plan and load discipline as the int8 kernel: the (tile, 32-row step) units dealt evenly to 8-wave
@@ -167,6 +164,7 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(int kst
         skinny_stash(total, m, wave, red);
     }
     const SkinnyScale no_scale;  // ones and no bias: the group scales are already in the totals
+    // (worked out here, not inside the loop: there it was measured to cost the loop more than it saves the tail)
     const SkinnyRoles roles = skinny_roles_of(plan, wk, grp, kSkinnyWaves);
     if (DT == HIDET_QMM_F16)
         skinny_tails<_Float16, kSkinnyWaves>(plan, wk, roles, m, n, no_scale, reinterpret_cast<_Float16 *>(c), mailbox, lost_flag, red);
@@ -218,7 +216,7 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
         return;
     }
     const Workspace ws = split_workspace(workspace, workspace_bytes);
-    const SkinnyPlan plan = skinny_make_plan(k, n, parallel_k_parts, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, QMM_W4_FLAT);
+    const SkinnyPlan plan = skinny_make_plan(k, n, parallel_k_parts, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, false, /*flat_ok=*/false, device_cus());
     // a wave's run of rows and the scale table are addressed with 31-bit offsets
     if ((cdiv(cdiv(skinny_units(plan), plan.groups), kSkinnyWaves) * 32 + 64) * (n / 2) >= (int64_t(1) << 31) - (1 << 20) ||
         (k / group) * n * 2 >= (int64_t(1) << 31) - (1 << 20)) {
@@ -230,7 +228,7 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     }
     // 16-byte activation loads through a buffer descriptor: aligned rows, offsets below 2^31
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16) && (15 * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
-    uint32_t *lost_flag = ws.counters != nullptr ? ws.counters + kSkinnyLostWord : nullptr;
+    uint32_t *lost_flag = ws.counters != nullptr ? ws.counters + kExchangeLostWord : nullptr;
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
         const size_t shmem = skinny_lds_bytes(mt, kSkinnyWaves);

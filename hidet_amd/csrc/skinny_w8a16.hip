@@ -179,7 +179,7 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, const 
     constexpr int waves = kWaves;
     const Workspace ws = split_workspace(workspace, workspace_bytes);
     SkinnyPlan plan;
-    if (fast) plan = skinny_make_plan(k, n, parallel_k_parts, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, strict_workspace);
+    if (fast) plan = skinny_make_plan(k, n, parallel_k_parts, int(std::min<int64_t>(16, m)), ws.mailbox_bytes, strict_workspace, /*flat_ok=*/true, device_cus());
     // a wave's run of rows is addressed with 31-bit offsets
     if (!fast || (cdiv(cdiv(skinny_units(plan), plan.groups), waves) * 32 + 160) * n >= (int64_t(1) << 31) - (1 << 20)) {
         launch(naive_w8a16_kernel, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, static_cast<const _Float16 *>(a), lda,
@@ -189,7 +189,7 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, const 
     }
     // 16-byte activation loads through a buffer descriptor: aligned rows, offsets below 2^31
     const bool aligned_a = (k % 8 == 0) && (lda % 8 == 0) && aligned(a, 16) && (15 * lda + k) * 2 < (int64_t(1) << 31) - (1 << 20);
-    uint32_t *lost_flag = ws.counters != nullptr ? ws.counters + kSkinnyLostWord : nullptr;
+    uint32_t *lost_flag = ws.counters != nullptr ? ws.counters + kExchangeLostWord : nullptr;
     for (int64_t m0 = 0; m0 < m; m0 += 16) {
         const int mt = int(std::min<int64_t>(16, m - m0));
         const _Float16 *ap = static_cast<const _Float16 *>(a) + m0 * lda;

@@ -17,6 +17,8 @@ LIB_PATH = os.path.join(_HERE, 'lib', 'libhidet_qmm.so')
 
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 
+ABI_VERSION = 2  # HIDET_QMM_ABI_VERSION of include/hidet_qmm.h
+
 # dtype codes of include/hidet_qmm.h
 F32, F16, BF16, I8, I16, E4M3, E5M2 = 0, 1, 2, 3, 4, 5, 6
 DTYPE_CODE = {
@@ -24,13 +26,16 @@ DTYPE_CODE = {
     torch.float8_e4m3fn: E4M3, torch.float8_e5m2: E5M2,
 }
 
-# name -> (restype, argtypes): every symbol include/hidet_qmm.h declares
+# name -> (restype, argtypes): every symbol include/hidet_qmm.h and include/hidet_qmm_bench.h declare
 SIGNATURES = {
     'hidet_set_last_error': (None, [ctypes.c_char_p]),
     'hidet_get_last_error': (ctypes.c_char_p, []),
     'hidet_qmm_abi_version': (_i32, []),
     'hidet_qmm_arch': (ctypes.c_char_p, []),
     'hidet_qmm_min_workspace_bytes': (_i64, []),
+    'hidet_qmm_workspace_bytes_for_scratch': (_i64, [_i64]),
+    'hidet_qmm_exchange_status': (_i32, [_vp, _i64, _vp]),
+    'hidet_qmm_exchange_reset': (None, [_vp, _i64, _vp]),
     'hidet_qmm_event_create': (_vp, []),
     'hidet_qmm_event_destroy': (None, [_vp]),
     'hidet_qmm_event_record': (None, [_vp, _vp]),
@@ -38,6 +43,8 @@ SIGNATURES = {
     'hidet_qmm_event_elapsed_ms': (_f32, [_vp, _vp]),
     'hidet_qmm_arm_timing': (None, [_vp, _vp]),
     'hidet_qmm_read_probe': (None, [_vp, _i64, _vp, _vp]),
+    'hidet_qmm_pattern_probe': (None, [_vp, _i64, _i64, _i32, _i32, _vp, _vp]),
+    'hidet_qmm_set_exchange_spin_limit': (None, [_i32]),
     'hidet_symmetric_quantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _i64, _vp]),
     'hidet_symmetric_dequantize': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _vp]),
     'hidet_symmetric_quant_matmul_f16_i8': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
@@ -72,8 +79,8 @@ def load_library() -> ctypes.CDLL:
         for name, (restype, argtypes) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = restype, argtypes
-        if lib.hidet_qmm_abi_version() != 1:
-            raise OSError('{} has ABI version {}, expected 1'.format(LIB_PATH, lib.hidet_qmm_abi_version()))
+        if lib.hidet_qmm_abi_version() != ABI_VERSION:
+            raise OSError('{} has ABI version {}, expected {}'.format(LIB_PATH, lib.hidet_qmm_abi_version(), ABI_VERSION))
         _LIB = lib
     return _LIB
 

@@ -20,8 +20,21 @@
  *     exchange split-K partial sums: the kernels leave every counter and every mailbox word they use at zero
  *     again.  The rest is plain scratch.  Two calls that overlap in time (different streams) must not share a
  *     workspace, and nothing else may write to one while a call is in flight.
+ *     In bytes: counters = 65536; mailbox = min(16 MiB, (workspace_bytes - 65536) / 4) rounded down to a multiple of 256;
+ *     scratch = workspace_bytes - 65536 - mailbox.  What each entry point needs of it:
+ *       hidet_symmetric_quantize          scratch >= 4 * outer * inner bytes (an error otherwise);
+ *       hidet_fp8_quantize_per_tensor     scratch >= 4 bytes (an error otherwise);
+ *       hidet_symmetric_quant_matmul_f16_i8[_bias], hidet_symmetric_quant_matmul_w4a16 with up to 16 rows
+ *                                         mailbox >= 1024 * min(m, 16) bytes per workgroup of the K split, at most 256
+ *                                         workgroups unless parallel_k_parts asks for more (4 MiB serve every automatic
+ *                                         plan); with less the kernels use fewer workgroups, never an error;
+ *       the same with more rows, hidet_matmul_f8, hidet_matmul_f8_scaled, the _nk matmuls
+ *                                         scratch: 64 KiB per tile computed in K ranges times the ranges (optional: with
+ *                                         less, fewer or no tiles are split; hidet_qmm_min_workspace_bytes() serves
+ *                                         every shape).
+ *     hidet_qmm_workspace_bytes_for_scratch(s) returns the smallest workspace whose scratch part holds s bytes.
  *
- * All tensors are dense row-major.  No function allocates device memory or synchronises.
+ * All tensors are dense row-major.  No function allocates device memory; none but hidet_qmm_exchange_status synchronises.
  */
 #ifndef HIDET_QMM_H
 #define HIDET_QMM_H
@@ -32,7 +45,9 @@
 extern "C" {
 #endif
 
-#define HIDET_QMM_ABI_VERSION 1
+/* 2: the workspace gained the mailbox (see above and hidet_qmm_workspace_bytes_for_scratch); measurement hooks moved to
+ * hidet_qmm_bench.h; hidet_qmm_exchange_status / hidet_qmm_exchange_reset added. */
+#define HIDET_QMM_ABI_VERSION 2
 
 /* element type codes */
 enum {
@@ -57,22 +72,22 @@ const char *hidet_qmm_arch(void);            /* "gfx950" */
 /* A workspace of this size lets every entry point use the K split it would choose for the shapes of a 4096- to 8192-wide
  * transformer; with less (or with very wide outputs) the kernels use fewer K slices, down to none, never an error. */
 int64_t hidet_qmm_min_workspace_bytes(void);
+/* The smallest workspace_bytes whose scratch part (what follows the counters and the mailbox) holds scratch_bytes. */
+int64_t hidet_qmm_workspace_bytes_for_scratch(int64_t scratch_bytes);
 
-/* ---- timing hook (measurement only) ----------------------------------------------------------
- * hidet_qmm_arm_timing makes the NEXT compute-kernel launch issued from this thread record its
- * own begin and end into the two events (the dispatch's timestamps, without launch gaps).  The
- * role of the reference's CompiledFunction.profile (python/hidet/runtime/compiled_module.py:106-147). */
-void *hidet_qmm_event_create(void);
-void hidet_qmm_event_destroy(void *event);
-void hidet_qmm_event_record(void *event, void *stream);
-void hidet_qmm_event_synchronize(void *event);
-float hidet_qmm_event_elapsed_ms(void *start, void *stop);
-void hidet_qmm_arm_timing(void *start_event, void *stop_event);
-/* Measurement only: one kernel that reads `bytes` (a multiple of 32768) from src with 16-byte loads, 32 KiB contiguous
- * per workgroup, and does nothing else (sink: 4 bytes of device memory, practically never written).  Timed through the
- * hook above it gives the rate at which this memory system delivers a matrix of that size to a kernel: the ceiling of
- * the decode kernels at their real sizes, next to the 8 TB/s of the data sheet.  No counterpart in the reference. */
-void hidet_qmm_read_probe(const void *src, int64_t bytes, void *sink, void *stream);
+/* ---- health of the split-K exchange ------------------------------------------------------------------
+ * The bandwidth-bound kernels sum their K slices through the workspace's mailbox: a workgroup that holds a column tile's
+ * last rows polls the mailbox for the partial tiles of the others.  The poll is bounded; if a partial tile never shows
+ * up (a workspace that was not zero-filled, two overlapping calls on one workspace, a device fault) the workgroup
+ * writes NaN to its outputs, sets a flag in the workspace and returns, and the mailbox may be left with stale words that
+ * would corrupt later calls.  No counterpart in the reference, whose split-K parts are separate outputs summed by a
+ * second operator (python/hidet/graph/ops/quant/resolve.py:99).
+ * hidet_qmm_exchange_status waits for `stream`, then returns 1 if any launch on this workspace gave up since the last
+ * reset, 0 if none did, -1 on an error (last-error string).  hidet_qmm_exchange_reset enqueues kernels on `stream` that
+ * zero the counters, the flag and the mailbox; call it after a status of 1, with no other call on the workspace in
+ * flight.  workspace == NULL names the current device's array of hidet_symmetric_quant_matmul_f16_i8_static. */
+int hidet_qmm_exchange_status(const void *workspace, int64_t workspace_bytes, void *stream);
+void hidet_qmm_exchange_reset(void *workspace, int64_t workspace_bytes, void *stream);
 
 /* ---- symmetric quantize / dequantize ---------------------------------------------------------
  * replaces the auto-scheduled kernels of SymmetricQuantizationTask / SymmetricDeQuantizationTask
@@ -117,7 +132,8 @@ void hidet_symmetric_quant_matmul_f16_i8_nk_bias(const void *a, const void *w_nk
  * needs more mailbox memory than the array's share of it (a quarter: 4 MiB) is rejected with an error that names the
  * bytes needed; taller matrices always run, in as many K ranges as fit the scratch part.  Every call on one GPU uses the same array: calls that overlap in
  * time on one GPU (two streams, two threads) race; calls ordered by a stream or by events do not.  The device the
- * stream belongs to must be current. */
+ * stream belongs to must be current.  The first call on a device looks up the array's address (hipGetSymbolAddress):
+ * make it outside any stream capture; later calls only launch kernels and may be captured. */
 #define HIDET_QMM_STATIC_SCRATCH_BYTES ((16 << 20) + (64 << 10))
 int64_t hidet_qmm_static_scratch_bytes(void);
 void hidet_symmetric_quant_matmul_f16_i8_static(const void *a, const void *w, const void *scale, void *c, int64_t m,

@@ -58,7 +58,7 @@ static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_par
 // each. Every unit must belong to exactly one wave, a workgroup's run may touch two tiles at most, every tile has one
 // collector (the workgroup with its last unit) that fetches exactly the slots of the workgroups before it in the tile,
 // every other contributor sends exactly once into its own slot, and the plan never needs more mailbox than there is.
-static int check_skinny(long long k, long long ncols, int hint, int rows, long long workspace_bytes) {
+static int check_skinny(long long k, long long ncols, int hint, int rows, long long workspace_bytes, bool flat_ok, int cus) {
     static char dummy[16];
     const Workspace ws = split_workspace(dummy, workspace_bytes);
     if (workspace_bytes >= kCounterBytes &&
@@ -66,22 +66,23 @@ static int check_skinny(long long k, long long ncols, int hint, int rows, long l
          kCounterBytes + ws.mailbox_bytes + ws.scratch_bytes != workspace_bytes ||
          reinterpret_cast<char *>(ws.mailbox) + ws.mailbox_bytes != ws.scratch))
         return std::printf("workspace of %lld bytes: mailbox %lld, scratch %lld\n", workspace_bytes, (long long)ws.mailbox_bytes, (long long)ws.scratch_bytes), 1;
-    const SkinnyPlan free_plan = skinny_make_plan(k, ncols, hint, rows, 1LL << 40, true);
+    const SkinnyPlan free_plan = skinny_make_plan(k, ncols, hint, rows, 1LL << 40, true, flat_ok, cus);
     const bool fits = skinny_mailbox_need(free_plan, rows) <= ws.mailbox_bytes;
     bool threw = false;
     try {
-        skinny_make_plan(k, ncols, hint, rows, ws.mailbox_bytes, true);
+        skinny_make_plan(k, ncols, hint, rows, ws.mailbox_bytes, true, flat_ok, cus);
     } catch (const Error &) { threw = true; }
     if (threw == fits) return std::printf("skinny k=%lld n=%lld rows=%d ws=%lld: strict error %d, fits %d\n", k, ncols, rows, workspace_bytes, threw, fits), 1;
-    const SkinnyPlan p = skinny_make_plan(k, ncols, hint, rows, ws.mailbox_bytes, false);
+    const SkinnyPlan p = skinny_make_plan(k, ncols, hint, rows, ws.mailbox_bytes, false, flat_ok, cus);
     if (fits && (p.groups != free_plan.groups)) return std::printf("skinny k=%lld n=%lld: a plan that fits was changed\n", k, ncols), 1;
     const int units = skinny_units(p);
     if (p.tiles != int((ncols + kSkinnyTileN - 1) / kSkinnyTileN) || p.ksteps != int((k + 31) / 32) || p.groups < p.tiles ||
         p.groups > units || p.groups > free_plan.groups || skinny_mailbox_need(p, rows) > ws.mailbox_bytes)
         return std::printf("skinny k=%lld n=%lld hint=%d rows=%d ws=%lld: %d tiles x %d steps, %d workgroups need %lld\n", k, ncols, hint, rows,
                            workspace_bytes, p.tiles, p.ksteps, p.groups, (long long)skinny_mailbox_need(p, rows)), 1;
-    if (hint == 0 && p.groups > 256 && p.groups != p.tiles)
-        return std::printf("skinny k=%lld n=%lld: %d workgroups do not fit one round\n", k, ncols, p.groups), 1;
+    if (hint == 0 && p.groups > std::min(cus, 256) && p.groups != p.tiles)
+        return std::printf("skinny k=%lld n=%lld: %d workgroups do not fit one round of %d CUs\n", k, ncols, p.groups, cus), 1;
+    if (!flat_ok && p.splits == 0) return std::printf("skinny k=%lld n=%lld: runs across tiles where whole slices were asked for\n", k, ncols), 1;
     constexpr int kWaves = 8;
     std::vector<int> seen(units, 0), collector(p.tiles, -1), first(p.tiles, -1), sends(p.groups, 0), sent_to(p.groups, -1);
     int most = 0;
@@ -172,8 +173,15 @@ int main() {
             for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL, 128256LL})
                 for (int rows : {1, 8, 16})
                     for (int hint : {0, 1, 3, 8, 64}) {
-                        if (check_skinny(k, nc, hint, rows, ws)) return 1;
-                        ++n;
+                        if (check_skinny(k, nc, hint, rows, ws, true, 256)) return 1;
+                        if (check_skinny(k, nc, hint, rows, ws, false, 256)) return 1;
+                        n += 2;
+                        // fewer CUs than a full device (a partition), more than the plan's cap
+                        if (hint == 0 && (ws == 0 || ws == (64LL << 20))) {
+                            for (int cus : {1, 32, 64, 80, 304})
+                                if (check_skinny(k, nc, hint, rows, ws, rows == 1, cus)) return 1;
+                            n += 5;
+                        }
                     }
     const int cfgs[][3] = {{32, 32, 4}, {32, 32, 8}, {64, 64, 4}, {64, 32, 4}};  // concurrent, fill, max_parts of the launchers
     for (const auto &c : cfgs)

@@ -15,10 +15,16 @@ from hidet_amd.graph.ops import quant
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
+HEADERS = ['hidet_qmm.h', 'hidet_qmm_bench.h']  # the operator ABI; measurement and test hooks
+
+
+def header_text():
+    text = ''.join(open(os.path.join(ROOT, 'include', h)).read() for h in HEADERS)
+    return re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+
+
 def declared_symbols():
-    text = open(os.path.join(ROOT, 'include', 'hidet_qmm.h')).read()
-    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
-    return sorted(set(re.findall(r'\b(hidet_[a-z0-9_]+)\s*\(', text)))
+    return sorted(set(re.findall(r'\b(hidet_[a-z0-9_]+)\s*\(', header_text())))
 
 
 def test_library_exports_every_declared_symbol():
@@ -29,7 +35,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
         assert name in ffi.SIGNATURES, 'no ctypes signature for ' + name
     assert sorted(ffi.SIGNATURES) == names
-    assert lib.hidet_qmm_abi_version() == 1
+    assert lib.hidet_qmm_abi_version() == 2 == ffi.ABI_VERSION
+    assert re.search(r'#define HIDET_QMM_ABI_VERSION 2\b', open(os.path.join(ROOT, 'include', 'hidet_qmm.h')).read())
     assert lib.hidet_qmm_arch() == b'gfx950'
     assert lib.hidet_qmm_min_workspace_bytes() >= (1 << 20)
 
@@ -121,8 +128,7 @@ def test_task_descriptions():
 
 def _declared_parameter_kinds():
     """name -> list of 'ptr' / 'i64' / 'i32' per parameter, parsed from the header's declarations."""
-    text = open(os.path.join(ROOT, 'include', 'hidet_qmm.h')).read()
-    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    text = header_text()
     out = {}
     for m in re.finditer(r'\b(hidet_[a-z0-9_]+)\s*\(([^)]*)\)\s*;', text):
         params = [p.strip() for p in m.group(2).split(',')]
@@ -156,9 +162,36 @@ def test_header_is_plain_c():
     gcc = shutil.which('gcc')
     if gcc is None:
         pytest.skip('gcc not available')
-    r = subprocess.run([gcc, '-std=c99', '-Wall', '-Werror', '-fsyntax-only', '-x', 'c', os.path.join(ROOT, 'include', 'hidet_qmm.h')],
-                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert r.returncode == 0, r.stdout
+    for h in HEADERS:
+        r = subprocess.run([gcc, '-std=c99', '-Wall', '-Werror', '-fsyntax-only', '-x', 'c', os.path.join(ROOT, 'include', h)],
+                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        assert r.returncode == 0, r.stdout
+
+
+def _workspace_parts(nbytes):
+    # the layout include/hidet_qmm.h states: counters, mailbox, scratch
+    if nbytes < 65536:
+        return 0, 0
+    rest = nbytes - 65536
+    mailbox = min(16 << 20, rest // 4) // 256 * 256
+    return mailbox, rest - mailbox
+
+
+def test_workspace_sizes_under_the_mailbox_layout():
+    lib = ffi.load_library()
+    for scratch in [0, 1, 4, 255, 256, 4096, 4 * 11008, 1 << 20, (48 << 20) - 1, 48 << 20, (48 << 20) + 1, 80 << 20, 1 << 30]:
+        need = lib.hidet_qmm_workspace_bytes_for_scratch(scratch)
+        assert _workspace_parts(need)[1] >= scratch, scratch
+        assert need == 65536 or _workspace_parts(need - 1)[1] < scratch, scratch  # and no byte more than that
+    # a workspace sized by the rule that held before the mailbox existed (64 KiB + the scale maxima) is now refused,
+    # with the bytes named; the size the helper gives passes this check (the call then stops at its null tensors)
+    nscale = 11008
+    old_rule = 65536 + 4 * nscale
+    lib.hidet_symmetric_quantize(1, 1, 1, 1, 4096, nscale, ffi.F32, ffi.I8, 256, old_rule, None)
+    msg = ffi.get_last_error()
+    assert msg is not None and 'workspace too small' in msg and str(4 * nscale) in msg
+    assert _workspace_parts(old_rule)[1] < 4 * nscale <= _workspace_parts(lib.hidet_qmm_workspace_bytes_for_scratch(4 * nscale))[1]
+    assert lib.hidet_qmm_min_workspace_bytes() >= lib.hidet_qmm_workspace_bytes_for_scratch(64 << 20)
 
 
 def test_int4_decode_layout_repacking():

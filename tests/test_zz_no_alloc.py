@@ -71,6 +71,50 @@ def test_static_scratch_matches_workspace_entry_point():
     assert np.array_equal(host(c1).view(np.uint16), host(c1b).view(np.uint16))
 
 
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph():
+    # device memory in use is the same before and after the calls (the library's side; the output tensors are made first)
+    a, q, s = _case(31, 1, 4096, 11008)
+    a2, q2, s2 = _case(32, 8, 2048, 1024)
+    d1 = [dev(x) for x in (a, q, s)]
+    d2 = [dev(x) for x in (a2, q2, s2)]
+    announce('static scratch: memory in use')
+    stream = ffi.current_stream(d1[0].device)
+    outs = [torch.empty((x[0].shape[0], x[1].shape[1]), dtype=torch.float16, device='cuda') for x in (d1, d2)]
+
+    def call(d, c):
+        ffi.call('hidet_symmetric_quant_matmul_f16_i8_static', d[0], d[1], d[2], c, d[0].shape[0], d[0].shape[1], d[1].shape[1],
+                 d[0].stride(0), 0, ffi.current_stream(d[0].device))
+
+    call(d1, outs[0])  # the first call on a device looks up the array's address: outside the measurement and any capture
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        call(d1, outs[0])
+        call(d2, outs[1])
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    eager = [host(o).copy() for o in outs]
+    assert ffi.call('hidet_qmm_exchange_status', None, 0, stream) == 0
+
+    # captured into a graph (the launches only: no allocation, no memset node), replayed with eager work in between
+    announce('static scratch: graph replays')
+    graph = torch.cuda.CUDAGraph()
+    g_outs = [torch.zeros_like(o) for o in outs]
+    with torch.cuda.graph(graph):
+        call(d1, g_outs[0])
+        call(d2, g_outs[1])
+    for rep in range(4):
+        for o in g_outs:
+            o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, e in zip(g_outs, eager):
+            assert np.array_equal(host(o).view(np.uint16), e.view(np.uint16)), rep
+        call(d2, outs[1])  # the program's own eager work between the replays, on the same array
+        torch.cuda.synchronize()
+        assert np.array_equal(host(outs[1]).view(np.uint16), eager[1].view(np.uint16))
+
+
 def test_static_scratch_exact_on_small_integers():
     rng = np.random.default_rng(5)
     for m, k, n, parts in [(5, 2048, 4096, 0), (2, 512, 256, 3), (16, 1024, 11008, 0)]:
