@@ -31,11 +31,24 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_FP8_PEAK_TFLOPS = 5000.0
-# HBM bytes one GEMV launch moves, from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over the --pmc-calibration
+# HBM bytes one GEMV launch moves come from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over the --pmc-calibration
 # run of this file, each scaled by what the same counter reads for a 64 MiB device copy. The figure is a record of that
-# profile, not measured in this run: it is reported together with the name of the summary it was taken from.
-GEMV_MEASURED_TRAFFIC_BYTES = 45.83e6
+# profile, not measured in this run: the summary keeps it in a small JSON block, which is read here and reported together
+# with the summary's name.
 GEMV_TRAFFIC_PROFILE = 'profiles/skinny_w8a16_gemv_m1_k4096_n11008_hbm_traffic.md'
+
+
+def measured_gemv_traffic():
+    """(bytes per launch or None, the record) from the ```json block of the traffic summary."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, GEMV_TRAFFIC_PROFILE)).read()
+        rec = json.loads(re.search(r'```json\s*(\{.*?\})\s*```', text, flags=re.S).group(1))
+        return float(rec['hbm_bytes_per_launch']), rec
+    except (OSError, AttributeError, KeyError, ValueError):
+        return None, None
+
+
 K, N = 4096, 11008
 RING = 16
 GEMV_BYTES = K * N + 2 * N + 2 * K + 2 * N  # weights + scales + activations + output, each once
@@ -289,6 +302,37 @@ def main():
     e1.synchronize()
     hot_us = e0.elapsed_time(e1) / 500 * 1e3
 
+    def time_gemm_series(launch_one, reps=24, skip=4):
+        """Kernel durations (us) of a GEMM, two ways, each started on a chip that has idled for a second (what ran before
+        in this process must not decide the clock a series gets). First `reps` launches back to back, each with its own
+        pair of events: the sustained rate, at whatever clock the chip holds under its power limit - the figure reported.
+        Then one launch at a time, each waited for before the next goes out: what a caller that consumes every result
+        before it asks for the next one sees (slower: every launch starts on an idle memory system)."""
+        def rest():
+            torch.cuda.synchronize()
+            time.sleep(1.0)
+        rest()
+        pairs = [(lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()) for _ in range(reps)]
+        for rep, (x0, x1) in enumerate(pairs):
+            lib.hidet_qmm_arm_timing(x0, x1)
+            launch_one(rep % 3)
+        stream.synchronize()
+        sustained = [lib.hidet_qmm_event_elapsed_ms(x0, x1) * 1e3 for x0, x1 in pairs]
+        for x0, x1 in pairs:
+            lib.hidet_qmm_event_destroy(x0)
+            lib.hidet_qmm_event_destroy(x1)
+        rest()
+        e0, e1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
+        one = []
+        for rep in range(reps):
+            lib.hidet_qmm_arm_timing(e0, e1)
+            launch_one(rep % 3)
+            lib.hidet_qmm_event_synchronize(e1)
+            one.append(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3)
+        lib.hidet_qmm_event_destroy(e0)
+        lib.hidet_qmm_event_destroy(e1)
+        return np.array(sustained[skip:]), np.array(one[skip:])
+
     # ---- second half of the metric: the M = 2048 prefill GEMM of the same weight shape ------------------------
     MP = 2048
     gp = torch.Generator(device=device)
@@ -306,16 +350,7 @@ def main():
     rows = np.array([0, 127, 128, 1029, 2047])
     pref = clib.quant_matmul_f32acc(ap.cpu().numpy()[rows], ws[2].cpu().numpy(), ss[2].cpu().numpy())
     prefill_parity = O.max_rel_err(cp.cpu().numpy()[rows], pref)
-    ev0, ev1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
-    pd = []
-    for rep in range(24):
-        lib.hidet_qmm_arm_timing(ev0, ev1)
-        launch_prefill(rep % RING)
-        lib.hidet_qmm_event_synchronize(ev1)
-        pd.append(lib.hidet_qmm_event_elapsed_ms(ev0, ev1) * 1e3)
-    lib.hidet_qmm_event_destroy(ev0)
-    lib.hidet_qmm_event_destroy(ev1)
-    pd = np.array(pd[4:])
+    pd, pd_single = time_gemm_series(launch_prefill)
     prefill_flops = 2.0 * MP * K * N
     prefill_tflops = prefill_flops / (pd.mean() * 1e-6) / 1e12
 
@@ -342,16 +377,7 @@ def main():
     ref8 = O.fp8_matmul_per_tensor(a8.view(torch.uint8).cpu().numpy()[rows8], b8s[2][0].view(torch.uint8).cpu().numpy(),
                                    float(sa.cpu()), float(b8s[2][1].cpu()), 'float32')
     fp8_parity = O.max_rel_err(c8.float().cpu().numpy()[rows8], ref8)
-    ev0, ev1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
-    fd = []
-    for rep in range(24):
-        lib.hidet_qmm_arm_timing(ev0, ev1)
-        launch_fp8(rep % 3)
-        lib.hidet_qmm_event_synchronize(ev1)
-        fd.append(lib.hidet_qmm_event_elapsed_ms(ev0, ev1) * 1e3)
-    lib.hidet_qmm_event_destroy(ev0)
-    lib.hidet_qmm_event_destroy(ev1)
-    fd = np.array(fd[4:])
+    fd, fd_single = time_gemm_series(launch_fp8)
     fp8_tflops = 2.0 * MF * KF * NF / (fd.mean() * 1e-6) / 1e12
 
     # ---- the other benchmark configurations, one figure each (kernel duration through the timing hook, distinct weight
@@ -436,6 +462,13 @@ def main():
     del wl
     us = time_kernel(lambda r: ffi.call('hidet_qmm_read_probe', ws[r % RING], K * N, sink, sptr), 64, 16)
     read_probe['read_only_kernel_45MB'] = hbm_entry(us, K * N)
+    # the loads of the GEMV kernel over the same matrices without its arithmetic and its exchange (256-column tiles, rows
+    # in steps of 32, one step per wave in flight), on the 256 workgroups of its launch and on the 172 of a plan of four
+    # slices per tile; and the same bytes per wave read as contiguous 1 KiB pieces
+    for label, groups, contiguous in (('gemv_access_pattern_256_workgroups', 256, 0), ('gemv_access_pattern_172_workgroups', 172, 0),
+                                      ('same_bytes_per_wave_contiguous_256_workgroups', 256, 1)):
+        us = time_kernel(lambda r: ffi.call('hidet_qmm_pattern_probe', ws[r % RING], K, N, groups, contiguous, sink, sptr), 64, 16)
+        read_probe[label + '_45MB'] = hbm_entry(us, K * N)
     # W8A16 prefill, attention QKV shape [2048, 4096] x [4096, 12288]
     wq = [torch.randint(-127, 128, (K, 12288), device=device, dtype=torch.int8) for _ in range(4)]
     sq = torch.cat([ss[0], ss[1]])[:12288].contiguous()
@@ -506,6 +539,7 @@ def main():
             'fp8_gemm_us': {'benchmark_operands': round(float(fd.mean()), 2), 'zero_operands': round(f8_zero, 2)}}}))
         return
 
+    traffic_bytes, traffic_record = measured_gemv_traffic()
     result = {
         'metric': 'w8a16_decode_gemv_bandwidth', 'value': round(value, 1), 'unit': 'GB/s', 'n_gpus': 1,
         'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 5), 'higher_is_better': True,
@@ -515,8 +549,8 @@ def main():
                    'launches_per_step': RING, 'distinct_weight_buffers': RING, 'bytes_per_launch': GEMV_BYTES,
                    'graph_replay': True},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': GEMV_MEASURED_TRAFFIC_BYTES,
-                     'traffic_source': GEMV_TRAFFIC_PROFILE, 'algorithmic_bytes': GEMV_BYTES,
+                     'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': traffic_bytes,
+                     'traffic_source': GEMV_TRAFFIC_PROFILE, 'traffic_record': traffic_record, 'algorithmic_bytes': GEMV_BYTES,
                      'duration_of': 'every launch of four laps of the ring, launched back to back behind one untimed lap, begin/end of its own dispatch',
                      'kernel': 'skinny_w8a16_kernel', 'kernel_us_mean': round(kernel_us, 3),
                      'kernel_us_min': round(float(durs.min()), 3), 'kernel_us_p50': round(float(np.median(durs)), 3),
@@ -525,13 +559,23 @@ def main():
                                   'GB/s': round(GEMV_BYTES / (hot_us * 1e-6) / 1e9, 1)},
         'prefill': {'workload': 'W8A16 prefill GEMM, a f16[2048,4096] x w int8[4096,11008] -> f16[2048,11008]',
                     'value': round(prefill_tflops, 1), 'unit': 'TFLOP/s', 'kernel': 'gemm_w8a16_kernel',
-                    'kernel_us_mean': round(float(pd.mean()), 2), 'kernel_us_min': round(float(pd.min()), 2),
+                    'kernel_us_mean': round(float(pd.mean()), 2), 'kernel_us_p50': round(float(np.median(pd)), 2),
+                    'kernel_us_min': round(float(pd.min()), 2),
+                    'timing': '20 launches back to back after a second of idle, begin/end of each dispatch',
+                    'one_launch_at_a_time': {'kernel_us_mean': round(float(pd_single.mean()), 2),
+                                             'TFLOP/s': round(prefill_flops / (pd_single.mean() * 1e-6) / 1e12, 1),
+                                             'frac': round(prefill_flops / (pd_single.mean() * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)},
                     'roofline': {'bound': 'mfma', 'achieved': round(prefill_tflops, 1), 'peak': MFMA_F16_PEAK_TFLOPS,
                                  'unit': 'TFLOP/s', 'frac': round(prefill_tflops / MFMA_F16_PEAK_TFLOPS, 4)},
                     'max_rel_err_vs_oracle_rows_sample': prefill_parity},
         'fp8_prefill': {'workload': 'FP8 e4m3 GEMM, a[4096,8192] x b[8192,8192]^T, per-tensor f32 scales -> bf16[4096,8192]',
                         'value': round(fp8_tflops, 1), 'unit': 'TFLOP/s', 'kernel': 'gemm_fp8_kernel',
-                        'kernel_us_mean': round(float(fd.mean()), 2), 'kernel_us_min': round(float(fd.min()), 2),
+                        'kernel_us_mean': round(float(fd.mean()), 2), 'kernel_us_p50': round(float(np.median(fd)), 2),
+                        'kernel_us_min': round(float(fd.min()), 2),
+                        'timing': '20 launches back to back after a second of idle, begin/end of each dispatch',
+                        'one_launch_at_a_time': {'kernel_us_mean': round(float(fd_single.mean()), 2),
+                                                 'TFLOP/s': round(2.0 * MF * KF * NF / (fd_single.mean() * 1e-6) / 1e12, 1),
+                                                 'frac': round(2.0 * MF * KF * NF / (fd_single.mean() * 1e-6) / 1e12 / MFMA_FP8_PEAK_TFLOPS, 4)},
                         'roofline': {'bound': 'mfma', 'achieved': round(fp8_tflops, 1), 'peak': MFMA_FP8_PEAK_TFLOPS,
                                      'unit': 'TFLOP/s', 'frac': round(fp8_tflops / MFMA_FP8_PEAK_TFLOPS, 4)},
                         'max_rel_err_vs_oracle_rows_sample': fp8_parity, 'tolerance': 3e-2},
