@@ -518,22 +518,12 @@ def main():
     del bring
 
     if args.data_dependence:
-        def timed(fn, reps=24):
-            e0, e1 = lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()
-            d = []
-            for rep in range(reps):
-                lib.hidet_qmm_arm_timing(e0, e1)
-                fn(rep)
-                lib.hidet_qmm_event_synchronize(e1)
-                d.append(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3)
-            lib.hidet_qmm_event_destroy(e0)
-            lib.hidet_qmm_event_destroy(e1)
-            return float(np.mean(d[4:]))
         az, wz = torch.zeros_like(ap), torch.zeros_like(ws[0])
         a8z, b8z = torch.zeros_like(a8.view(torch.uint8)), torch.zeros_like(b8s[0][0].view(torch.uint8))
-        w8_zero = timed(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', az, wz, ss[0], cp, MP, K, N, K, 0, work,
-                                           work.numel(), sptr))
-        f8_zero = timed(lambda r: ffi.call('hidet_matmul_f8', a8z, b8z, c8, MF, NF, KF, KF, KF, 2, sa, b8s[0][1], work, work.numel(), sptr))
+        w8_zero = float(time_gemm_series(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', az, wz, ss[0], cp, MP, K, N, K, 0, work,
+                                                            work.numel(), sptr))[0].mean())
+        f8_zero = float(time_gemm_series(lambda r: ffi.call('hidet_matmul_f8', a8z, b8z, c8, MF, NF, KF, KF, KF, 2, sa, b8s[0][1], work,
+                                                            work.numel(), sptr))[0].mean())
         print(json.dumps({'data_dependence': {
             'w8a16_gemm_us': {'benchmark_operands': round(float(pd.mean()), 2), 'zero_operands': round(w8_zero, 2)},
             'fp8_gemm_us': {'benchmark_operands': round(float(fd.mean()), 2), 'zero_operands': round(f8_zero, 2)}}}))

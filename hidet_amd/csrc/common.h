@@ -201,4 +201,14 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
 
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) { return static_cast<float>(__builtin_bit_cast(_Float16, b)); }
 
+// The float16 output of the int8 matmul with the optional bias of its epilogue: the product is rounded to float16 and the
+// bias is added to that value with a second rounding - what the reference's fused epilogue computes, which applies the add
+// to the value the template stores (python/hidet/graph/ops/quant/matmul_f16_i8.py:95-99) - so a fused call and the
+// matmul followed by an add give the same bits. `bias` of a call without one is -0.0f, which changes nothing (not even
+// the sign of a zero).
+__device__ __forceinline__ _Float16 scaled_biased_f16(float acc, float scale, float bias) {
+    const _Float16 product = _Float16(acc * scale);
+    return _Float16(float(product) + bias);
+}
+
 }  // namespace qmm

@@ -288,7 +288,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         sc[t] = float(scale[col + t]);
-        bs[t] = bias != nullptr ? float(bias[col + t]) : 0.0f;
+        bs[t] = bias != nullptr ? float(bias[col + t]) : -0.0f;
     }
 #pragma unroll
     for (int rb = 0; rb < RBA; ++rb)
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(WM * WN * 64, MIN_BLOCKS) void gemm_w8a16_kernel16(
             if (row < m) {
                 half4_t o;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) o[t] = _Float16(fmaf(acc[rb][t][v], sc[t], bs[t]));
+                for (int t = 0; t < 4; ++t) o[t] = scaled_biased_f16(acc[rb][t][v], sc[t], bs[t]);
                 *reinterpret_cast<half4_t *>(c + int64_t(row) * n + col) = o;
             }
         }

@@ -2,6 +2,8 @@
 // workgroup split its run of 32-row steps): the launch plan, the LDS reduction over the waves and the exchange of
 // partial tiles between workgroups.
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace qmm {
@@ -310,14 +312,20 @@ struct SkinnyTail {
         }
         return r;
     }
+    // one output element: float16 outputs take the column factor and the bias (two roundings, see scaled_biased_f16);
+    // bfloat16 outputs have neither (the int4 kernel folds its group scales in before)
+    __device__ __forceinline__ OutT finish(float sum, int e) const {
+        if constexpr (std::is_same<OutT, _Float16>::value) return scaled_biased_f16(sum, scale[e], bias[e]);
+        else return skinny_to_out<OutT>(sum);
+    }
     __device__ __forceinline__ void store(int row, const Vals &x) const {
         OutT *dst = c + int64_t(row) * n + out_col;
         if constexpr (CW == 1) {
-            dst[0] = skinny_to_out<OutT>(fmaf(x.v[0], scale[0], bias[0]));
+            dst[0] = finish(x.v[0], 0);
         } else {
             uint16_t h[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, skinny_to_out<OutT>(fmaf(x.v[e], scale[e], bias[e])));
+            for (int e = 0; e < 4; ++e) h[e] = __builtin_bit_cast(uint16_t, finish(x.v[e], e));
             // 8 bytes at once when the row starts allow it (n a multiple of 4 is given, the base pointer may not be aligned)
             if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
                 *reinterpret_cast<uint2 *>(dst) = uint2{uint32_t(h[0]) | (uint32_t(h[1]) << 16), uint32_t(h[2]) | (uint32_t(h[3]) << 16)};
@@ -358,7 +366,7 @@ struct SkinnyTail {
 #pragma unroll
         for (int e = 0; e < CW; ++e) {
             scale[e] = factors.scale != nullptr ? f16_bits_to_f32(uint16_t(scale_bits[e >> 1] >> (16 * (e & 1)))) : 1.0f;
-            bias[e] = f16_bits_to_f32(uint16_t(bias_bits[e >> 1] >> (16 * (e & 1))));
+            bias[e] = factors.bias != nullptr ? f16_bits_to_f32(uint16_t(bias_bits[e >> 1] >> (16 * (e & 1)))) : -0.0f;
         }
     }
 
@@ -394,7 +402,8 @@ struct SkinnyTail {
             return;
         }
         // a trip: one output row of this thread and up to 8 or 16 slots (two rows of 8 slots per trip were measured
-        // slower than two trips: 16 rows at 4096 x 11008 16.3 against 14.2 us)
+        // slower than two trips: 16 rows at 4096 x 11008 16.3 against 14.2 us); with at most 4 slots to fetch - whole
+        // slices per tile - a trip takes two or four of the thread's rows, which costs no more than one
         if (roles.fetch_others > 8) collect<1, 16>(mailbox, roles, send_slot);
         else if (roles.fetch_others <= 4 && m > 2 * kRowGroups) collect<4, 4>(mailbox, roles, send_slot);
         else if (roles.fetch_others <= 4 && m > kRowGroups) collect<2, 4>(mailbox, roles, send_slot);
@@ -593,7 +602,9 @@ constexpr int kSkinnyPlanWaves = 8;          // waves of a workgroup of the kern
 constexpr int kSkinnyMinUnitsPerGroup = 2 * kSkinnyPlanWaves;  // two 32-row steps per wave
 // The runs ignore the tile boundaries up to this many activation rows and while a tile has no more than this many
 // contributors; beyond, whole runs per tile with a tile's runs on one XCD are faster (one row at 11008 x 4096, 16 tiles:
-// 12.4 against 10.4 us; 16 rows at 4096 x 4096: 12.0 against 10.4 us).
+// 12.4 against 10.4 us; 16 rows at 4096 x 4096: 12.0 against 10.4 us; 4 and 8 rows at 4096 x 11008: 12.7 and 13.5 against
+// 12.4 and 13.2 us). The int4 kernel always takes whole runs per tile: its matrix is half the bytes, and the exchange
+// with five or six senders per tile cost it more than the idle CUs of four slices (one row: 10.0 against 9.6 us).
 constexpr int kSkinnyFlatRows = 2, kSkinnyFlatSharers = 8;
 
 // Bytes of mailbox a plan touches: one fp32 partial tile of `rows` (at most 16) activation rows per workgroup, slot =

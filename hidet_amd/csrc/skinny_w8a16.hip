@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256) void naive_w8a16_kernel(const _Float16 *__rest
     const int64_t i = o / n, j = o - i * n;
     float acc = 0.f;
     for (int64_t kk = 0; kk < k; ++kk) acc += float(a[i * lda + kk]) * float(w[kk * n + j]);
-    c[o] = _Float16(fmaf(acc, float(scale[j]), bias != nullptr ? float(bias[j]) : 0.0f));
+    c[o] = scaled_biased_f16(acc, float(scale[j]), bias != nullptr ? float(bias[j]) : -0.0f);
 }
 
 }  // namespace

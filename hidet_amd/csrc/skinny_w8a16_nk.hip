@@ -144,7 +144,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_kernel(const _Floa
         float v = 0.f;
 #pragma unroll
         for (int p = 0; p < WAVES; ++p) v += red[p][row][cn];
-        c[int64_t(row) * n + n0 + cn] = _Float16(fmaf(v, float(scale[n0 + cn]), bias != nullptr ? float(bias[n0 + cn]) : 0.0f));
+        c[int64_t(row) * n + n0 + cn] = scaled_biased_f16(v, float(scale[n0 + cn]), bias != nullptr ? float(bias[n0 + cn]) : -0.0f);
     }
 }
 
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_nk_wide_kernel(const 
             float v = 0.f;
 #pragma unroll
             for (int p = 0; p < WAVES; ++p) v += red[p][g][row][cn];
-            c[int64_t(row) * n + col] = _Float16(fmaf(v, float(scale[col]), bias != nullptr ? float(bias[col]) : 0.0f));
+            c[int64_t(row) * n + col] = scaled_biased_f16(v, float(scale[col]), bias != nullptr ? float(bias[col]) : -0.0f);
         }
     }
 }

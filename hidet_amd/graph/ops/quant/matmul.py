@@ -154,7 +154,8 @@ def symmetric_quant_matmul(a: torch.Tensor, weight: torch.Tensor, scale: torch.T
                            bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The reference's operator (python/hidet/graph/ops/quant/matmul.py:83-93).  `bias`, which the reference's signature
     does not have, is the fused form of the epilogue its template admits (matmul_f16_i8.py:95-99): a float16 [N] vector
-    added to the fp32 result before the one rounding to float16."""
+    added to the float16 result (two roundings, as the reference's fused epilogue and the matmul followed by an add
+    give): fused and unfused calls return the same bits."""
     signature = (a.shape, a.dtype, weight.shape, weight.dtype, scale.shape, scale.dtype,
                  None if bias is None else (bias.shape, bias.dtype))
     if signature in _VALIDATED:

@@ -24,8 +24,10 @@ class SymmetricQuantizedMatmulF16I8Task(Task):
         return False
 
     def allow_epilogue(self) -> bool:
-        # the reference's template accepts fused epilogues; the pre-built kernels do not
-        return False
+        # as in the reference (matmul_f16_i8.py:98-99). What the pre-built kernels can take into their epilogue is the bias
+        # add of a linear layer (the rewrite rule SymmetricQuantizeMatmulBiasFused); any other consumer stays an operator
+        # of its own
+        return True
 
 
 class SymmetricQuantizedMatmulF16I8Op(Operator):

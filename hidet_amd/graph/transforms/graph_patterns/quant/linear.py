@@ -200,7 +200,8 @@ class SymmetricQuantizeMatmulBiasFused(SubgraphRewriteRule):
     """add(symmetric_quant_matmul(x, wq, scale), bias) => symmetric_quant_matmul(x, wq, scale, bias) for a constant float16
     bias of one element per output column: the bias of an nn.Linear rides in the kernel's epilogue instead of a separate
     element-wise launch per layer. The reference gets the same effect from its fusion pass, which folds the add into the
-    template's epilogue (matmul_f16_i8.py:95-99, allow_epilogue); there is no rule of this name there."""
+    template's epilogue (matmul_f16_i8.py:95-99, allow_epilogue); there is no rule of this name there. The fused kernel adds
+    the bias to the float16 product with a second rounding, so the rewritten graph returns the bits of the unfused one."""
 
     def __init__(self):
         super().__init__('add(fused_matmulf16(x, wq, scale), bias) => fused_matmulf16(x, wq, scale, bias)')

@@ -113,8 +113,9 @@ void hidet_symmetric_dequantize(const void *wq, const void *scale, void *w, int6
 void hidet_symmetric_quant_matmul_f16_i8(const void *a, const void *w, const void *scale, void *c, int64_t m,
                                          int64_t k, int64_t n, int64_t lda, int parallel_k_parts, void *workspace,
                                          int64_t workspace_bytes, void *stream);
-/* The same two operators with the bias of a linear layer added in the epilogue: c = cast(acc * scale[n] + bias[n]) with one
- * rounding, bias float16 [n] (NULL: none).  No counterpart in the reference's operator signature; it is the fused form of
+/* The same two operators with the bias of a linear layer added in the epilogue: c = f16(f16(acc * scale[n]) + bias[n]),
+ * the bits the matmul followed by a float16 add gives (the reference's fused epilogue adds to the stored float16 value
+ * as well); bias float16 [n] (NULL: none).  No counterpart in the reference's operator signature; it is the fused form of
  * the epilogue the reference's template admits (allow_epilogue, python/hidet/graph/ops/quant/matmul_f16_i8.py:95-99), so
  * that a rewritten nn.Linear with bias is one launch. */
 void hidet_symmetric_quant_matmul_f16_i8_bias(const void *a, const void *w, const void *scale, const void *bias, void *c,

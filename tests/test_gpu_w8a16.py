@@ -103,23 +103,47 @@ def test_split_k_parts_api_and_hints():
                                           (12, 512, 8200, 'kn'), (40, 2048, 520, 'kn'), (300, 512, 1100, 'kn'), (2, 100, 40, 'kn'),
                                           (1, 4096, 1024, 'nk'), (16, 1024, 512, 'nk'), (40, 2048, 520, 'nk'), (12, 8192, 8192, 'nk')])
 def test_bias_in_the_epilogue_exact(m, k, n, layout):
-    # c = acc * scale + bias with one rounding: integer operands, power-of-two scales and a bias of small multiples of
-    # 2^-10 make every step exact in fp32; every kernel family that has the epilogue (both tail layouts of the
+    # c = f16(f16(acc * scale) + bias): integer operands, power-of-two scales and a bias of small multiples of
+    # 2^-10 make every step exact; every kernel family that has the epilogue (both tail layouts of the
     # bandwidth-bound kernel, the MFMA GEMM, the element-wise fallback, the kernels for K-contiguous weights)
     announce('w8a16 bias', m, k, n, layout)
     a, q, s = _int_case(m * 7 + n, m, k, n)
     rng = np.random.default_rng(n)
     b = (rng.integers(-64, 65, n) / 1024.0).astype(np.float16)
-    want = (a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :] + b.astype(np.float64)[None, :]
+    product = ((a.astype(np.int64) @ q.astype(np.int64)).astype(np.float64) * s.astype(np.float64)[None, :]).astype(np.float32).astype(np.float16)
+    want = (product.astype(np.float32) + b.astype(np.float32)[None, :]).astype(np.float16)
     tq = dev(q)
     if layout == 'nk':
         tq = quant.to_decode_layout(tq)
     got = host(quant.symmetric_quant_matmul(dev(a), tq, dev(s), dev(b)))
-    assert np.array_equal(got, want.astype(np.float32).astype(np.float16))
+    assert np.array_equal(got, want)
     plain = host(quant.symmetric_quant_matmul(dev(a), tq, dev(s)))  # the same call without bias is unchanged
-    assert np.array_equal(plain, (want - b.astype(np.float64)[None, :]).astype(np.float32).astype(np.float16))
+    assert np.array_equal(plain, product)
     with pytest.raises(ValueError, match='bias must be'):
         quant.symmetric_quant_matmul(dev(a), tq, dev(s), dev(b[:-1]))
+
+
+@pytest.mark.parametrize('m,k,n,layout', [(1, 4096, 11008, 'kn'), (8, 2048, 4096, 'kn'), (16, 1024, 768, 'kn'), (40, 2048, 520, 'kn'),
+                                          (300, 512, 1100, 'kn'), (2, 100, 40, 'kn'), (1, 4096, 1024, 'nk'), (16, 1024, 512, 'nk'),
+                                          (40, 2048, 520, 'nk')])
+def test_fused_bias_gives_the_bits_of_matmul_then_add(m, k, n, layout):
+    # random operands, where one rounding and two differ in the last bit of some outputs: the fused epilogue rounds the
+    # scaled sum to float16 and adds the bias to that (python/hidet/graph/ops/quant/matmul_f16_i8.py:95-99: the reference's
+    # epilogue fusion applies the add to the value the template stores), so it equals the unfused pair bit for bit
+    announce('w8a16 fused bias == matmul + add', m, k, n, layout)
+    a32, w32 = O.make_inputs(m * 11 + n, m, k, n)
+    q, s32 = O.symmetric_quantize(w32, 'int8', dims=0)
+    a, s = a32.astype(np.float16), s32.astype(np.float16)
+    b = (np.random.default_rng(n).standard_normal(n) * 0.5).astype(np.float16)
+    tq = dev(q)
+    if layout == 'nk':
+        tq = quant.to_decode_layout(tq)
+    fused = host(quant.symmetric_quant_matmul(dev(a), tq, dev(s), dev(b)))
+    plain = host(quant.symmetric_quant_matmul(dev(a), tq, dev(s)))
+    want = (plain.astype(np.float32) + b.astype(np.float32)[None, :]).astype(np.float16)  # a float16 add, rounded once
+    assert np.array_equal(fused.view(np.uint16), want.view(np.uint16))
+    single = (clib.quant_matmul_f32acc(a, q, s).astype(np.float64))  # sanity: the bias really changed something
+    assert not np.array_equal(fused, plain) and single.shape == fused.shape
 
 
 @pytest.mark.parametrize('m,k,n,parts', [(2, 8192, 16384, 32), (16, 4096, 8192, 16), (1, 16384, 4096, 64)])
