@@ -288,6 +288,17 @@ def main():
         lib.hidet_qmm_event_destroy(e1)
     durs = np.array(durs[LAPS * RING:])  # first pass warms the instruction cache
     kernel_us = float(durs.mean())
+    # where the slow launches are: by weight buffer (physical placement of a 45 MB buffer), by position in a pass
+    # (a pass starts behind one untimed lap), by pass
+    by_launch = durs.reshape(-1, LAPS, RING)
+    slow = durs > 1.2 * np.median(durs)
+    spread = {'p90': round(float(np.percentile(durs, 90)), 3), 'p99': round(float(np.percentile(durs, 99)), 3),
+              'max': round(float(durs.max()), 3),
+              'mean_by_weight_buffer': [round(float(x), 2) for x in by_launch.mean(axis=(0, 1))],
+              'mean_by_lap_of_a_pass': [round(float(x), 2) for x in by_launch.mean(axis=(0, 2))],
+              'mean_by_pass': [round(float(x), 2) for x in by_launch.mean(axis=(1, 2))],
+              'launches_over_1.2_x_p50': int(slow.sum()),
+              'of_them_by_weight_buffer': [int(x) for x in slow.reshape(-1, LAPS, RING).sum(axis=(0, 1))]}
     achieved = GEMV_BYTES / (kernel_us * 1e-6) / 1e9
 
     # single-buffer (last-level-cache-hot) figure, labelled as such
@@ -544,7 +555,7 @@ def main():
                      'duration_of': 'every launch of four laps of the ring, launched back to back behind one untimed lap, begin/end of its own dispatch',
                      'kernel': 'skinny_w8a16_kernel', 'kernel_us_mean': round(kernel_us, 3),
                      'kernel_us_min': round(float(durs.min()), 3), 'kernel_us_p50': round(float(np.median(durs)), 3),
-                     'launches_timed': int(durs.size)},
+                     'launches_timed': int(durs.size), 'spread_us': spread},
         'llc_hot_single_buffer': {'us_per_launch_back_to_back': round(hot_us, 3),
                                   'GB/s': round(GEMV_BYTES / (hot_us * 1e-6) / 1e9, 1)},
         'prefill': {'workload': 'W8A16 prefill GEMM, a f16[2048,4096] x w int8[4096,11008] -> f16[2048,11008]',
