@@ -9,13 +9,14 @@ void gemm_fp8_launch(const void *a, const void *b, void *c, int64_t m, int64_t n
                      int out_dtype, const void *scale_a, const void *scale_b, void *workspace, int64_t workspace_bytes,
                      hipStream_t stream);
 void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                            int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream);
+                            int64_t n, int64_t k, int out_dtype, bool e5m2, void *workspace, int64_t workspace_bytes,
+                            hipStream_t stream);
 void skinny_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
                             int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
 void gemm_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, int64_t n, int64_t k, int64_t lda, int64_t ldb,
                           int out_dtype, const void *scale_a, const void *scale_b, hipStream_t stream);
 void skinny_fp8_block_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                                    int64_t n, int64_t k, int out_dtype, hipStream_t stream);
+                                    int64_t n, int64_t k, int out_dtype, bool e5m2, hipStream_t stream);
 }  // namespace qmm
 
 using namespace qmm;
@@ -69,11 +70,14 @@ HIDET_API void hidet_matmul_f8_e5m2(const void *a, const void *b, void *c, int64
     QMM_ENTRY_END
 }
 
-HIDET_API void hidet_matmul_f8_scaled(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c,
-                                      int64_t m, int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes,
-                                      void *stream_) {
-    QMM_ENTRY_BEGIN
-    check_out_dtype(out_dtype);
+// Checks and kernel choice of the block-scaled matmul; `e5m2`: both operands float8_e5m2, else float8_e4m3.
+static void f8_scaled_dispatch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m, int64_t n,
+                               int64_t k, int out_dtype, bool e5m2, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+    if (e5m2)
+        QMM_CHECK(out_dtype == HIDET_QMM_F32 || out_dtype == HIDET_QMM_F16 || out_dtype == HIDET_QMM_BF16 || out_dtype == HIDET_QMM_E5M2,
+                  "output dtype must be float32, float16, bfloat16 or float8_e5m2, got code " << out_dtype);
+    else
+        check_out_dtype(out_dtype);
     QMM_CHECK(m >= 0 && n >= 0 && k >= 0, "negative extent: m=" << m << " n=" << n << " k=" << k);
     QMM_CHECK(k % 128 == 0 && n % 128 == 0,
               "block-scaled matmul needs K and N to be multiples of the 128 x 128 scale block, got K=" << k << " N=" << n);
@@ -84,8 +88,23 @@ HIDET_API void hidet_matmul_f8_scaled(const void *a, const void *b, const void *
     QMM_CHECK(aligned(a, 16) && aligned(b, 16) && aligned(c, 16), "tensors must be 16-byte aligned");
     check_workspace(workspace, workspace_bytes);
     if (m <= 16)  // decode: the bandwidth-bound kernel, one pass over b
-        skinny_fp8_block_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, static_cast<hipStream_t>(stream_));
+        skinny_fp8_block_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, e5m2, stream);
     else
-        gemm_fp8_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
+        gemm_fp8_scaled_launch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, e5m2, workspace, workspace_bytes, stream);
+}
+
+HIDET_API void hidet_matmul_f8_scaled(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c,
+                                      int64_t m, int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes,
+                                      void *stream_) {
+    QMM_ENTRY_BEGIN
+    f8_scaled_dispatch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, false, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
+    QMM_ENTRY_END
+}
+
+HIDET_API void hidet_matmul_f8_scaled_e5m2(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c,
+                                           int64_t m, int64_t n, int64_t k, int out_dtype, void *workspace,
+                                           int64_t workspace_bytes, void *stream_) {
+    QMM_ENTRY_BEGIN
+    f8_scaled_dispatch(a, b, scale_a, scale_b, c, m, n, k, out_dtype, true, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
     QMM_ENTRY_END
 }

@@ -27,6 +27,32 @@ constexpr int kChunksPerThread = kStageChunks / kThreads;  // 8
 constexpr int kLdsBytes = 2 * kStageChunks * 16;           // 64 KiB
 
 template <int OUT>
+__device__ __forceinline__ void store4_scaled(void *c, int64_t o, float4_t v) {
+    if (OUT == HIDET_QMM_F32) {
+        *reinterpret_cast<float4_t *>(static_cast<float *>(c) + o) = v;
+    } else if (OUT == HIDET_QMM_BF16) {
+        uint2 w2;
+        w2.x = uint32_t(f32_to_bf16_bits(v[0])) | (uint32_t(f32_to_bf16_bits(v[1])) << 16);
+        w2.y = uint32_t(f32_to_bf16_bits(v[2])) | (uint32_t(f32_to_bf16_bits(v[3])) << 16);
+        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
+    } else if (OUT == HIDET_QMM_F16) {
+        uint2 w2;
+        w2.x = uint32_t(f32_to_f16_bits(v[0])) | (uint32_t(f32_to_f16_bits(v[1])) << 16);
+        w2.y = uint32_t(f32_to_f16_bits(v[2])) | (uint32_t(f32_to_f16_bits(v[3])) << 16);
+        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
+    } else if (OUT == HIDET_QMM_E5M2) {
+        *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(c) + o) =
+            uint32_t(f32_to_e5m2(v[0])) | (uint32_t(f32_to_e5m2(v[1])) << 8) | (uint32_t(f32_to_e5m2(v[2])) << 16) |
+            (uint32_t(f32_to_e5m2(v[3])) << 24);
+    } else {
+        *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(c) + o) =
+            uint32_t(f32_to_e4m3(v[0])) | (uint32_t(f32_to_e4m3(v[1])) << 8) | (uint32_t(f32_to_e4m3(v[2])) << 16) |
+            (uint32_t(f32_to_e4m3(v[3])) << 24);
+    }
+}
+
+// FMT: operand format of the MFMA, 0 = float8 e4m3, 1 = float8 e5m2 (both operands the same).
+template <int OUT, int FMT = 0>
 __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_scaled_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
                                                                       const float *__restrict__ scale_a,
                                                                       const float *__restrict__ scale_b, void *__restrict__ c,
@@ -107,7 +133,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_scaled_kernel(const uint
                 rv[0] = int(bf[j][0].x); rv[1] = int(bf[j][0].y); rv[2] = int(bf[j][0].z); rv[3] = int(bf[j][0].w);
                 rv[4] = int(bf[j][1].x); rv[5] = int(bf[j][1].y); rv[6] = int(bf[j][1].z); rv[7] = int(bf[j][1].w);
                 const float4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    rv, cv, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+                    rv, cv, float4_t{0.f, 0.f, 0.f, 0.f}, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) total[i][j][v] += part[v] * f[i];
             }
@@ -126,23 +152,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_scaled_kernel(const uint
             if (col >= n) continue;
             const int64_t o = int64_t(row) * n + col;
             const float4_t v = total[i][j];
-            if (OUT == HIDET_QMM_F32) {
-                *reinterpret_cast<float4_t *>(static_cast<float *>(c) + o) = v;
-            } else if (OUT == HIDET_QMM_BF16) {
-                uint2 w2;
-                w2.x = uint32_t(f32_to_bf16_bits(v[0])) | (uint32_t(f32_to_bf16_bits(v[1])) << 16);
-                w2.y = uint32_t(f32_to_bf16_bits(v[2])) | (uint32_t(f32_to_bf16_bits(v[3])) << 16);
-                *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
-            } else if (OUT == HIDET_QMM_F16) {
-                uint2 w2;
-                w2.x = uint32_t(f32_to_f16_bits(v[0])) | (uint32_t(f32_to_f16_bits(v[1])) << 16);
-                w2.y = uint32_t(f32_to_f16_bits(v[2])) | (uint32_t(f32_to_f16_bits(v[3])) << 16);
-                *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
-            } else {
-                *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(c) + o) =
-                    uint32_t(f32_to_e4m3(v[0])) | (uint32_t(f32_to_e4m3(v[1])) << 8) | (uint32_t(f32_to_e4m3(v[2])) << 16) |
-                    (uint32_t(f32_to_e4m3(v[3])) << 24);
-            }
+            store4_scaled<OUT>(c, o, v);
         }
     }
 }
@@ -157,36 +167,16 @@ constexpr int kLoads8 = kSlotChunks8 / kThreads8;  // 6 direct-to-LDS loads per 
 constexpr int kRingBytes8 = 3 * kSlotChunks8 * 16;  // 144 KiB
 constexpr int kLdsBytes8 = kRingBytes8 + 16;       // + the K-split fix-up's flag; the ring must start at LDS address 0
 
-template <int OUT>
-__device__ __forceinline__ void store4_scaled(void *c, int64_t o, float4_t v) {
-    if (OUT == HIDET_QMM_F32) {
-        *reinterpret_cast<float4_t *>(static_cast<float *>(c) + o) = v;
-    } else if (OUT == HIDET_QMM_BF16) {
-        uint2 w2;
-        w2.x = uint32_t(f32_to_bf16_bits(v[0])) | (uint32_t(f32_to_bf16_bits(v[1])) << 16);
-        w2.y = uint32_t(f32_to_bf16_bits(v[2])) | (uint32_t(f32_to_bf16_bits(v[3])) << 16);
-        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
-    } else if (OUT == HIDET_QMM_F16) {
-        uint2 w2;
-        w2.x = uint32_t(f32_to_f16_bits(v[0])) | (uint32_t(f32_to_f16_bits(v[1])) << 16);
-        w2.y = uint32_t(f32_to_f16_bits(v[2])) | (uint32_t(f32_to_f16_bits(v[3])) << 16);
-        *reinterpret_cast<uint2 *>(static_cast<uint16_t *>(c) + o) = w2;
-    } else {
-        *reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(c) + o) =
-            uint32_t(f32_to_e4m3(v[0])) | (uint32_t(f32_to_e4m3(v[1])) << 8) | (uint32_t(f32_to_e4m3(v[2])) << 16) |
-            (uint32_t(f32_to_e4m3(v[3])) << 24);
-    }
-}
-
+template <int FMT>
 __device__ __forceinline__ float4_t mfma_fp8_k128_fresh(const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1) {
     const int8v_t rv = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
     const int8v_t cv = __builtin_shufflevector(c0, c1, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, float4_t{0.f, 0.f, 0.f, 0.f}, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
 
 // SCALED: scale_a / scale_b are the block scales described at the top of the file. !SCALED: plain a x b^T with optional
 // per-tensor scales (one float each, may be null), applied to the sums in the epilogue.
-template <int OUT, bool SCALED>
+template <int OUT, bool SCALED, int FMT = 0>
 __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *__restrict__ a, int64_t lda,
                                                                  const uint8_t *__restrict__ b, int64_t ldb,
                                                                  const float *__restrict__ scale_a,
@@ -342,11 +332,11 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
         lds_wait_keep_newer<12>(bf[0][0], bf[0][1]);
         lds_wait_keep_newer<12>(af[0][0], af[0][1]);
         auto mm = [&](float4_t &dst_scaled, float4_t &dst_plain, const int4v_t &r0, const int4v_t &r1, const int4v_t &c0, const int4v_t &c1) {
-            if constexpr (SCALED) dst_scaled = mfma_fp8_k128_fresh(r0, r1, c0, c1);
+            if constexpr (SCALED) dst_scaled = mfma_fp8_k128_fresh<FMT>(r0, r1, c0, c1);
             else {
                 const int8v_t rv = __builtin_shufflevector(r0, r1, 0, 1, 2, 3, 4, 5, 6, 7);
                 const int8v_t cv = __builtin_shufflevector(c0, c1, 0, 1, 2, 3, 4, 5, 6, 7);
-                dst_plain = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, dst_plain, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+                dst_plain = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, dst_plain, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
             }
         };
         mm(part[0][0], total[0][0], bf[0][0], bf[0][1], af[0][0], af[0][1]);
@@ -431,7 +421,7 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_fp8_kernel8(const uint8_t *
 
 // Launch of the 8-wave kernel; SCALED selects block scales (scale_a [K/128, M], scale_b [N/128, K/128]) or optional
 // per-tensor scales.
-template <bool SCALED>
+template <bool SCALED, int FMT = 0>
 static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ldb, const void *scale_a, const void *scale_b,
                            void *c, int64_t m, int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes,
                            hipStream_t stream) {
@@ -455,13 +445,12 @@ static void launch_kernel8(const void *a, int64_t lda, const void *b, int64_t ld
                int(m), int(n), int(k), tiles_m, tiles_n, tiling.xm, tiling.xn, tail.parts, tail.max_tiles,
                reinterpret_cast<float *>(ws.scratch), ws.counters);
     };
-    switch (out_dtype) {
-        case HIDET_QMM_F32: go(gemm_fp8_kernel8<HIDET_QMM_F32, SCALED>); break;
-        case HIDET_QMM_F16: go(gemm_fp8_kernel8<HIDET_QMM_F16, SCALED>); break;
-        case HIDET_QMM_BF16: go(gemm_fp8_kernel8<HIDET_QMM_BF16, SCALED>); break;
-        case HIDET_QMM_E4M3: go(gemm_fp8_kernel8<HIDET_QMM_E4M3, SCALED>); break;
-        default: QMM_FAIL("unsupported output dtype code " << out_dtype);
-    }
+    constexpr int kOut8 = FMT == 1 ? HIDET_QMM_E5M2 : HIDET_QMM_E4M3;  // the 8-bit output type is the operands' own
+    if (out_dtype == HIDET_QMM_F32) go(gemm_fp8_kernel8<HIDET_QMM_F32, SCALED, FMT>);
+    else if (out_dtype == HIDET_QMM_F16) go(gemm_fp8_kernel8<HIDET_QMM_F16, SCALED, FMT>);
+    else if (out_dtype == HIDET_QMM_BF16) go(gemm_fp8_kernel8<HIDET_QMM_BF16, SCALED, FMT>);
+    else if (out_dtype == kOut8) go(gemm_fp8_kernel8<kOut8, SCALED, FMT>);
+    else QMM_FAIL("unsupported output dtype code " << out_dtype);
 }
 
 // a x b^T with optional per-tensor scales on the 256 x 128, 8-wave kernel. The caller has checked: K a multiple of 128,
@@ -472,12 +461,13 @@ void gemm_fp8_kernel8_launch(const void *a, const void *b, void *c, int64_t m, i
     launch_kernel8<false>(a, lda, b, ldb, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
 }
 
-void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                            int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
+template <int FMT>
+static void scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m, int64_t n,
+                          int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, hipStream_t stream) {
     const bool fast = m * k <= (int64_t(1) << 30) && n * k <= (int64_t(1) << 30) && (k / 128) * m * 4 < (int64_t(1) << 31) &&
                       aligned(a, 16) && aligned(b, 16) && aligned(c, 16);
     if (fast) {
-        launch_kernel8<true>(a, k, b, k, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
+        launch_kernel8<true, FMT>(a, k, b, k, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
         return;
     }
     const int tiles_m = int(cdiv(m, kT)), tiles_n = int(n / 128);
@@ -488,13 +478,20 @@ void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, c
                static_cast<const uint8_t *>(b), static_cast<const float *>(scale_a), static_cast<const float *>(scale_b), c,
                int(m), int(n), int(k), tiles_m);
     };
-    switch (out_dtype) {
-        case HIDET_QMM_F32: go(gemm_fp8_scaled_kernel<HIDET_QMM_F32>); break;
-        case HIDET_QMM_F16: go(gemm_fp8_scaled_kernel<HIDET_QMM_F16>); break;
-        case HIDET_QMM_BF16: go(gemm_fp8_scaled_kernel<HIDET_QMM_BF16>); break;
-        case HIDET_QMM_E4M3: go(gemm_fp8_scaled_kernel<HIDET_QMM_E4M3>); break;
-        default: QMM_FAIL("unsupported output dtype code " << out_dtype);
-    }
+    constexpr int kOut8 = FMT == 1 ? HIDET_QMM_E5M2 : HIDET_QMM_E4M3;
+    if (out_dtype == HIDET_QMM_F32) go(gemm_fp8_scaled_kernel<HIDET_QMM_F32, FMT>);
+    else if (out_dtype == HIDET_QMM_F16) go(gemm_fp8_scaled_kernel<HIDET_QMM_F16, FMT>);
+    else if (out_dtype == HIDET_QMM_BF16) go(gemm_fp8_scaled_kernel<HIDET_QMM_BF16, FMT>);
+    else if (out_dtype == kOut8) go(gemm_fp8_scaled_kernel<kOut8, FMT>);
+    else QMM_FAIL("unsupported output dtype code " << out_dtype);
+}
+
+// `e5m2`: both operands are float8_e5m2 (the 8-bit output type is then e5m2 as well), else e4m3.
+void gemm_fp8_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
+                            int64_t n, int64_t k, int out_dtype, bool e5m2, void *workspace, int64_t workspace_bytes,
+                            hipStream_t stream) {
+    if (e5m2) scaled_launch<1>(a, b, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
+    else scaled_launch<0>(a, b, scale_a, scale_b, c, m, n, k, out_dtype, workspace, workspace_bytes, stream);
 }
 
 }  // namespace qmm

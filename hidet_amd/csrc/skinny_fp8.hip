@@ -105,7 +105,8 @@ __global__ __launch_bounds__(256) void skinny_fp8_kernel(const uint8_t *__restri
 // and 128 output columns): every step's products are accumulated from zero and added to the total times both factors.
 // The 16 row factors of a step are fetched by the 16 lanes of a group like one more operand and turned into the four
 // each lane needs (rows 4 kg .. 4 kg + 3) through LDS, per step, as the activations are.
-template <int OUT, int WAVES, bool BLOCK_SCALED = false>
+// FMT: operand format of the MFMA, 0 = float8 e4m3, 1 = float8 e5m2.
+template <int OUT, int WAVES, bool BLOCK_SCALED = false, int FMT = 0>
 __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uint8_t *__restrict__ a, int64_t lda,
                                                                 const uint8_t *__restrict__ b, int64_t ldb,
                                                                 void *__restrict__ c, int m, int n, int k,
@@ -167,11 +168,11 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
                 float *ft = reinterpret_cast<float *>(factor_stage[wave][d & 1]);
                 ft[ls] = fr[d];  // the four lane groups store the same 16 values
                 const float4_t f = factor_stage[wave][d & 1][kg];
-                const float4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, zero, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+                const float4_t part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, zero, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) acc[v] = fmaf(part[v], f[v], acc[v]);
             } else {
-                acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+                acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rv, cv, acc, FMT, FMT, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
             }
         }
     }
@@ -189,6 +190,7 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_fp8_staged_kernel(const uin
         if (OUT == HIDET_QMM_F32) static_cast<float *>(c)[o] = v;
         else if (OUT == HIDET_QMM_BF16) static_cast<uint16_t *>(c)[o] = f32_to_bf16_bits(v);
         else if (OUT == HIDET_QMM_F16) static_cast<uint16_t *>(c)[o] = f32_to_f16_bits(v);
+        else if (OUT == HIDET_QMM_E5M2) static_cast<uint8_t *>(c)[o] = f32_to_e5m2(v);
         else static_cast<uint8_t *>(c)[o] = f32_to_e4m3(v);
     }
 }
@@ -248,7 +250,7 @@ void skinny_fp8_e5m2_launch(const void *a, const void *b, void *c, int64_t m, in
 // Block-scaled operands (scale_a f32 [K/128, M], scale_b f32 [N/128, K/128]), up to 16 rows, contiguous a [M, K] and b [N, K],
 // K and N multiples of 128, everything 16-byte aligned (the entry point checks that).
 void skinny_fp8_block_scaled_launch(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
-                                    int64_t n, int64_t k, int out_dtype, hipStream_t stream) {
+                                    int64_t n, int64_t k, int out_dtype, bool e5m2, hipStream_t stream) {
     const uint8_t *ap = static_cast<const uint8_t *>(a), *bp = static_cast<const uint8_t *>(b);
     const float *sa = static_cast<const float *>(scale_a), *sb = static_cast<const float *>(scale_b);
     const dim3 grid(uint32_t(cdiv(n, 16)));
@@ -256,15 +258,25 @@ void skinny_fp8_block_scaled_launch(const void *a, const void *b, const void *sc
     auto go = [&](auto kern, int waves) {
         launch(kern, grid, dim3(64 * waves), 0, stream, ap, k, bp, k, c, int(m), int(n), int(k), sa, sb);
     };
-#define QMM_FP8_SKINNY_SCALED(OUT)                                          \
-    if (eight) go(skinny_fp8_staged_kernel<OUT, 8, true>, 8);               \
-    else go(skinny_fp8_staged_kernel<OUT, 4, true>, 4);
-    switch (out_dtype) {
-        case HIDET_QMM_F32: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F32) break;
-        case HIDET_QMM_F16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F16) break;
-        case HIDET_QMM_BF16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_BF16) break;
-        case HIDET_QMM_E4M3: QMM_FP8_SKINNY_SCALED(HIDET_QMM_E4M3) break;
-        default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+#define QMM_FP8_SKINNY_SCALED(OUT, FMT)                                     \
+    if (eight) go(skinny_fp8_staged_kernel<OUT, 8, true, FMT>, 8);          \
+    else go(skinny_fp8_staged_kernel<OUT, 4, true, FMT>, 4);
+    if (e5m2) {  // both operands float8_e5m2; the 8-bit output type is the operands' own
+        switch (out_dtype) {
+            case HIDET_QMM_F32: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F32, 1) break;
+            case HIDET_QMM_F16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F16, 1) break;
+            case HIDET_QMM_BF16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_BF16, 1) break;
+            case HIDET_QMM_E5M2: QMM_FP8_SKINNY_SCALED(HIDET_QMM_E5M2, 1) break;
+            default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+        }
+    } else {
+        switch (out_dtype) {
+            case HIDET_QMM_F32: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F32, 0) break;
+            case HIDET_QMM_F16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_F16, 0) break;
+            case HIDET_QMM_BF16: QMM_FP8_SKINNY_SCALED(HIDET_QMM_BF16, 0) break;
+            case HIDET_QMM_E4M3: QMM_FP8_SKINNY_SCALED(HIDET_QMM_E4M3, 0) break;
+            default: QMM_FAIL("unsupported output dtype code " << out_dtype);
+        }
     }
 #undef QMM_FP8_SKINNY_SCALED
 }

@@ -60,6 +60,7 @@ SIGNATURES = {
     'hidet_matmul_f8': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _i64, _vp]),
     'hidet_matmul_f8_e5m2': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp]),
     'hidet_matmul_f8_scaled': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
+    'hidet_matmul_f8_scaled_e5m2': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
 }
 
 

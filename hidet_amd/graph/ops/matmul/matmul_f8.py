@@ -3,8 +3,8 @@
 `hidet_matmul_f8_scaled`, plus the per-tensor quantize / matmul pair of the benchmark configuration.
 
 A is [..., M, K] and B is [..., N, K], both K-major, both float8_e4m3 or both float8_e5m2 (OCP formats, the MFMA's
-fp8 and bf8 operand types).  The e4m3 path has the tuned kernels; e5m2 runs the unscaled matmul on plainer ones, and
-the block-scaled matmul is built for e4m3 only."""
+fp8 and bf8 operand types).  The e4m3 path has the tuned kernels; e5m2 runs the unscaled matmul on plainer ones and
+the block-scaled matmul on the same kernels as e4m3 (`hidet_matmul_f8_scaled_e5m2`)."""
 from typing import List, Optional, Tuple
 
 import torch
@@ -138,7 +138,8 @@ class MatmulF8ScaledOperator(Operator):
         c = torch.empty((a3.shape[0], m, n), dtype=out, device=a.device)
         ws = ffi.workspace(a.device)
         for i in range(a3.shape[0]):
-            ffi.call('hidet_matmul_f8_scaled', a3[i], b3[i], sa3[i], sb3[i], c[i], m, n, k, ffi.DTYPE_CODE[out],
+            ffi.call('hidet_matmul_f8_scaled_e5m2' if a.dtype == f8e5m2 else 'hidet_matmul_f8_scaled', a3[i], b3[i], sa3[i], sb3[i],
+                     c[i], m, n, k, ffi.DTYPE_CODE[out],
                      ws, ws.numel(), ffi.current_stream(a.device))
         return [c.reshape(head + (a.shape[-2], n))]
 
@@ -176,8 +177,6 @@ def _matmul_f8(a, b, is_scaled: bool, scale_a=None, scale_b=None, bias=None, acc
         raise ValueError('a and b must have at least 2 dimensions, got shape {} and {}'.format(list(a.shape), list(b.shape)))
     if (a.dtype != f8e4m3 or b.dtype != f8e4m3) and (a.dtype != f8e5m2 or b.dtype != f8e5m2):
         raise ValueError('matmul_f8 only supports both operands being f8e4m3 or f8e5m2, got {} and {}'.format(a.dtype, b.dtype))
-    if a.dtype == f8e5m2 and is_scaled:
-        raise NotImplementedError('block-scaled matmul is built for float8_e4m3 operands only')
     signature = (a.shape, a.dtype, b.shape, b.dtype, acc_dtype, output_dtype)  # as the caller passed them
     if output_dtype is None:
         output_dtype = a.dtype

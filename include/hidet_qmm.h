@@ -208,6 +208,12 @@ void hidet_matmul_f8_e5m2(const void *a, const void *b, void *c, int64_t m, int6
  * scale_b float32 [n/128, k/128]; a [m, k] and b [n, k] dense. */
 void hidet_matmul_f8_scaled(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
                             int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, void *stream);
+/* The same task for float8_e5m2 operands (MatmulF8ScaledTask asserts only that both operands have the same dtype,
+ * python/hidet/graph/ops/matmul/matmul_f8.py:386-389, and _matmul_f8 admits both-e5m2 for the scaled form too, :709-712):
+ * same arguments and meaning; out_dtype float8_e5m2, float16, bfloat16 or float32. Same kernels with the MFMA's bf8
+ * operand format. */
+void hidet_matmul_f8_scaled_e5m2(const void *a, const void *b, const void *scale_a, const void *scale_b, void *c, int64_t m,
+                                 int64_t n, int64_t k, int out_dtype, void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

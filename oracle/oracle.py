@@ -412,11 +412,15 @@ def matmul_f8(a_code: np.ndarray, b_code: np.ndarray, out_dtype: Union[str, None
     return _cast_out(c, out_dtype)
 
 
-def matmul_f8_scaled(a_code, b_code, scale_a, scale_b, out_dtype: str = 'bfloat16', block: int = 128) -> np.ndarray:
+def matmul_f8_scaled(a_code, b_code, scale_a, scale_b, out_dtype: str = 'bfloat16', block: int = 128,
+                     in_dtype: str = 'float8_e4m3') -> np.ndarray:
     """Per K-block of 128: C += (sum_{k in blk} A*B) * scale_a[kb, m] * scale_b[nb, kb]
-    (matmul_f8.py:357-363, 632-636); scale_a is [K/128, M], scale_b is [N/128, K/128]."""
-    a = e4m3_decode(a_code)
-    b = e4m3_decode(b_code)
+    (matmul_f8.py:357-363, 632-636); scale_a is [K/128, M], scale_b is [N/128, K/128]. Both operands are of
+    `in_dtype`, float8_e4m3 or float8_e5m2 (the task asserts only that they agree, :386-389; _matmul_f8 admits both
+    formats for the scaled form as well, :709-712)."""
+    decode = e5m2_decode if in_dtype == 'float8_e5m2' else e4m3_decode
+    a = decode(a_code)
+    b = decode(b_code)
     m, k = a.shape
     n = b.shape[0]
     c = np.zeros((m, n), dtype=np.float32)

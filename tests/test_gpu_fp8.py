@@ -149,6 +149,56 @@ def test_matmul_f8_scaled_parity_real_scales(m, k, n):
     assert err <= 1e-4, err  # fp32 accumulation on both sides: only the order of the sums differs
 
 
+@pytest.mark.parametrize('a_shape, b_shape', [[[2048, 256], [4096, 256]], [[100, 384], [256, 384]], [[40, 4096], [1024, 4096]],
+                                              [[500, 7168], [1536, 7168]], [[1, 7168], [1536, 7168]], [[16, 4096], [4096, 4096]],
+                                              [[5, 384], [256, 384]], [[3, 128], [128, 128]]])
+def test_matmul_f8_scaled_e5m2_reference_recipe(a_shape, b_shape):
+    # the scaled task takes both operands float8_e5m2 as well (matmul_f8.py:386-389, 709-712): the recipe of
+    # tests/operators_core/test_matmul.py:291-373 on e5m2 codes - integers in [-4, 4] and integer scales are exact in e5m2 -
+    # through every kernel of the scaled path (8-wave tiles with and without K ranges, the bandwidth-bound kernel)
+    announce('matmul_f8_scaled e5m2', a_shape, b_shape)
+    rng = np.random.default_rng(43)
+    (m, k), n = a_shape, b_shape[0]
+    ai = rng.integers(-4, 5, a_shape)
+    bi = rng.integers(-4, 5, b_shape)
+    sa = rng.integers(1, 5, (k // 128, m)).astype(np.float32)
+    sb = rng.integers(1, 5, (n // 128, k // 128)).astype(np.float32)
+    ac, bc = O.e5m2_encode(ai.astype(np.float32)), O.e5m2_encode(bi.astype(np.float32))
+    assert np.array_equal(O.e5m2_decode(ac), ai) and np.array_equal(O.e5m2_decode(bc), bi)
+    ta, tb = dev(ac).view(torch.float8_e5m2), dev(bc).view(torch.float8_e5m2)
+    got = F8.matmul_f8_scaled(ta, tb, scale_a=dev(sa), scale_b=dev(sb), output_dtype='float32')
+    a2 = ai.astype(np.int64) * np.repeat(sa.T.astype(np.int64), 128, axis=1)
+    b2 = bi.astype(np.int64) * np.repeat(np.repeat(sb.astype(np.int64), 128, axis=0), 128, axis=1)
+    exact = (a2.astype(np.float64) @ b2.astype(np.float64).T).astype(np.int64)
+    assert np.array_equal(host(got).astype(np.int64), exact)
+    gotb = F8.matmul_f8_scaled(ta, tb, scale_a=dev(sa), scale_b=dev(sb), output_dtype='bfloat16')
+    assert np.array_equal(host(gotb), O.to_bf16(exact.astype(np.float32)))
+    got8 = F8.matmul_f8_scaled(ta, tb, scale_a=dev(sa), scale_b=dev(sb))  # default: the operands' own type
+    assert got8.dtype == torch.float8_e5m2
+    assert np.array_equal(got8.view(torch.uint8).cpu().numpy(), O.e5m2_encode(exact.astype(np.float32)))
+    with pytest.raises(ValueError, match='unsupported output dtype'):
+        F8.matmul_f8_scaled(ta, tb, scale_a=dev(sa), scale_b=dev(sb), output_dtype=torch.float8_e4m3fn)
+    if m <= 128:
+        ref = O.matmul_f8_scaled(ac, bc, sa, sb, 'float32', in_dtype='float8_e5m2')
+        assert np.array_equal(host(got), ref)
+
+
+@pytest.mark.parametrize('m,k,n', [(1, 4096, 4096), (16, 2048, 8192), (40, 1024, 512), (300, 512, 768)])
+def test_matmul_f8_scaled_e5m2_parity_real_scales(m, k, n):
+    # random e5m2 codes (subnormals and large magnitudes included) and real-valued block scales against the oracle
+    announce('matmul_f8_scaled e5m2 real scales', m, k, n)
+    rng = np.random.default_rng(m + k + 1)
+    ac = O.e5m2_encode((rng.standard_normal((m, k)) * np.exp2(rng.integers(-16, 3, (m, k)))).astype(np.float32))
+    bc = O.e5m2_encode((rng.standard_normal((n, k)) * 0.5).astype(np.float32))
+    sa = rng.uniform(0.5, 2.0, (k // 128, m)).astype(np.float32)
+    sb = rng.uniform(0.01, 0.05, (n // 128, k // 128)).astype(np.float32)
+    got = F8.matmul_f8_scaled(dev(ac).view(torch.float8_e5m2), dev(bc).view(torch.float8_e5m2), scale_a=dev(sa), scale_b=dev(sb),
+                              output_dtype='float32')
+    ref = O.matmul_f8_scaled(ac, bc, sa, sb, 'float32', in_dtype='float8_e5m2')
+    err = O.max_rel_err(host(got), ref)
+    assert err <= 1e-4, err  # fp32 accumulation on both sides: only the order of the sums differs
+
+
 @pytest.mark.parametrize('m,k,n', [(1, 8192, 8192), (16, 1024, 512), (256, 512, 768), (4096, 8192, 8192), (33, 400, 260)])
 def test_per_tensor_parity(m, k, n):
     announce('fp8 per-tensor', m, k, n)
@@ -341,8 +391,8 @@ def test_argument_errors():
         F8.matmul_f8(a[0], a)
     with pytest.raises(ValueError, match=r'\[\.\.\.,M,K\] and \[\.\.\.,N,K\]'):
         F8.matmul_f8(a, torch.zeros(4, 32, device='cuda').to(torch.float8_e4m3fn))
-    with pytest.raises(NotImplementedError):
-        F8.matmul_f8_scaled(a.to(torch.float8_e5m2), a.to(torch.float8_e5m2), torch.ones(1, 4, device='cuda'), torch.ones(1, 1, device='cuda'))
+    with pytest.raises(ValueError, match='only supports both operands'):  # mixed formats, scaled form
+        F8.matmul_f8_scaled(a, a.to(torch.float8_e5m2), torch.ones(1, 4, device='cuda'), torch.ones(1, 1, device='cuda'))
     with pytest.raises(ValueError, match='unsupported output dtype'):
         F8.matmul_f8(a, a, output_dtype='float8_e5m2')
     with pytest.raises(ValueError, match='bias is not supported'):

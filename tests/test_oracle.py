@@ -446,6 +446,24 @@ def test_matmul_f8_scaled_reference_recipe():
     assert np.array_equal(got.astype(np.int64), a2 @ b2.T)
 
 
+def test_matmul_f8_scaled_e5m2_reference_recipe():
+    # the same recipe on float8_e5m2 codes (both operands e5m2: matmul_f8.py:386-389, 709-712); integers up to 4 and the
+    # integer scales are exact in e5m2, so the pre-multiplied integer product pins the decode and the block indexing
+    rng = np.random.default_rng(43)
+    m, n, k = 48, 256, 384
+    ai = rng.integers(-4, 5, (m, k))
+    bi = rng.integers(-4, 5, (n, k))
+    sa = rng.integers(1, 5, (k // 128, m)).astype(np.float32)
+    sb = rng.integers(1, 5, (n // 128, k // 128)).astype(np.float32)
+    ac, bc = O.e5m2_encode(ai.astype(np.float32)), O.e5m2_encode(bi.astype(np.float32))
+    got = O.matmul_f8_scaled(ac, bc, sa, sb, out_dtype='float32', in_dtype='float8_e5m2')
+    a2 = ai.astype(np.int64) * np.repeat(sa.T.astype(np.int64), 128, axis=1)
+    b2 = bi.astype(np.int64) * np.repeat(np.repeat(sb.astype(np.int64), 128, axis=0), 128, axis=1)
+    assert np.array_equal(got.astype(np.int64), a2 @ b2.T)
+    # the same bytes read as e4m3 are other numbers: the format argument is not ignored
+    assert not np.array_equal(O.matmul_f8_scaled(ac, bc, sa, sb, out_dtype='float32'), got)
+
+
 def test_e5m2_codec_against_torch_and_float16():
     # decode: every code against torch.float8_e5m2 and against "upper byte of the float16 of the same value"
     codes = np.arange(256, dtype=np.uint8)
