@@ -10,9 +10,17 @@ import torch
 
 from hidet_amd import option
 
-# The reference estimates 80 SMs x 5 resident blocks (resolve.py:46); an MI355X has 256 CUs and the
-# streaming kernel runs one round of one 8-wave workgroup on each.
-ESTIMATE_CONCURRENT_BLOCKS = 256
+# The reference estimates 80 SMs x 5 resident blocks (resolve.py:46); here the streaming kernel runs one round of one
+# 8-wave workgroup per CU, and the library sizes its own plan for the CUs of the device it launches on (at most 256,
+# a full MI355X).
+MAX_CONCURRENT_BLOCKS = 256
+
+
+def estimate_concurrent_blocks(device=None) -> int:
+    """Workgroups the streaming kernel keeps in flight on `device`: one per CU, at most 256 (what the library's plan uses)."""
+    if not torch.cuda.is_available():
+        return MAX_CONCURRENT_BLOCKS
+    return min(MAX_CONCURRENT_BLOCKS, int(torch.cuda.get_device_properties(device).multi_processor_count))
 SEARCH_CANDIDATES = [1, 2, 3, 4, 5, 6, 8, 10, 12, 16]  # resolve.py:54
 
 
@@ -39,7 +47,7 @@ def resolve_parallel_k_parts(parallel_k: Union[str, int], a: torch.Tensor, b: to
     """Hint passed to the library for `symmetric_quant_matmul`.
 
     'disabled' (the reference's default) and 'default' leave the split to the library's own plan, which is
-    sized for 256 CUs; an integer is passed through clamped to [1, 32] as in the reference; 'search' times the
+    sized for the CUs of the device (`estimate_concurrent_blocks`); an integer is passed through clamped to [1, 32] as in the reference; 'search' times the
     reference's candidate list on the GPU and keeps the fastest.
     """
     if isinstance(parallel_k, str):
