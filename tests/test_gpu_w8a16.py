@@ -31,7 +31,12 @@ def _int_case(seed, m, k, n):
 
 @pytest.mark.parametrize('m,k,n', [(1, 256, 256), (1, 4096, 512), (3, 1024, 768), (16, 512, 256), (7, 96, 48),
                                    (1, 40, 16), (2, 8, 16), (1, 4096, 272), (16, 4096, 4096),
-                                   (9, 4096, 8192), (16, 1024, 11008), (12, 512, 8200)])  # 9 to 16 rows on wide outputs
+                                   (9, 4096, 8192), (16, 1024, 11008), (12, 512, 8200),  # 9 to 16 rows on wide outputs
+                                   # one and two rows on at least 32 column tiles: runs of (tile, step) units across the tiles -
+                                   # the headline shape, K not a multiple of 32, a last tile of 16 columns, fewer runs than CUs,
+                                   # a long K on few tiles, two contributors per tile, as many tiles as runs (nothing exchanged)
+                                   (1, 4096, 11008), (2, 4096, 11008), (1, 1000, 8208), (2, 544, 12288), (1, 96, 16400),
+                                   (1, 11008, 8192), (2, 2080, 32768), (2, 2080, 65536), (3, 4096, 11008)])
 def test_exact_on_small_integers(m, k, n):
     # integer activations and codes with power-of-two scales: every product and partial sum is exact in
     # fp32, so any dropped row, wrong byte or lost K slice shows as a whole-number difference
