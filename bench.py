@@ -273,14 +273,20 @@ def main():
     # ---- the kernel's own duration: begin/end of every dispatch through the timing hook, the ring launched back to
     # back as in the timed region (each launch has its own pair of events; one synchronisation per pass) -------------
     LAPS = 4  # the ring this many times per pass, back to back: 64 consecutive launches between two synchronisations
+    import ctypes
     evs = [(lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()) for _ in range(LAPS * RING)]
+    ptr_array = ctypes.c_void_p * RING
+    ev_array = ctypes.c_void_p * (LAPS * RING)
+    w_ptrs, s_ptrs, o_ptrs = (ptr_array(*[t.data_ptr() for t in ts]) for ts in (ws, ss, outs))
+    e0s, e1s = ev_array(*[e[0] for e in evs]), ev_array(*[e[1] for e in evs])
     durs = []
     for rep in range(5):
-        for i in range(RING):  # untimed: the pass starts behind a synchronisation, the timed region does not
-            launch(i, sptr)
-        for j in range(LAPS * RING):
-            lib.hidet_qmm_arm_timing(evs[j][0], evs[j][1])
-            launch(j % RING, sptr)
+        # one native loop per pass: an untimed lap (the pass starts behind a synchronisation, the timed region does not),
+        # then the timed launches. Issued from Python one call at a time, a launch costs the host about as long as the
+        # kernel runs, and on a slow host the stream's queue runs dry in the later laps of a pass: the kernels then start
+        # on an idle memory system and take 0.5-1.5 us longer (seen as a mean that grows from lap to lap)
+        ffi.call('hidet_qmm_gemv_ring_timed', a, w_ptrs, s_ptrs, o_ptrs, RING, RING, 1, K, N, K, work, work.numel(), None, None, sptr)
+        ffi.call('hidet_qmm_gemv_ring_timed', a, w_ptrs, s_ptrs, o_ptrs, RING, LAPS * RING, 1, K, N, K, work, work.numel(), e0s, e1s, sptr)
         stream.synchronize()
         durs.extend(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3 for e0, e1 in evs)
     for e0, e1 in evs:
@@ -552,7 +558,7 @@ def main():
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': traffic_bytes,
                      'traffic_source': GEMV_TRAFFIC_PROFILE, 'traffic_record': traffic_record, 'algorithmic_bytes': GEMV_BYTES,
-                     'duration_of': 'every launch of four laps of the ring, launched back to back behind one untimed lap, begin/end of its own dispatch',
+                     'duration_of': 'every launch of four laps of the ring, launched back to back from one native loop behind one untimed lap, begin/end of its own dispatch',
                      'kernel': 'skinny_w8a16_kernel', 'kernel_us_mean': round(kernel_us, 3),
                      'kernel_us_min': round(float(durs.min()), 3), 'kernel_us_p50': round(float(np.median(durs)), 3),
                      'launches_timed': int(durs.size), 'spread_us': spread},

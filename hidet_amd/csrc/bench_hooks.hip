@@ -44,6 +44,24 @@ HIDET_API void hidet_qmm_arm_timing(void *start_event, void *stop_event) {
     ts.stop = static_cast<hipEvent_t>(stop_event);
 }
 
+HIDET_API void hidet_qmm_gemv_ring_timed(const void *a, const void *const *weights, const void *const *scales, void *const *outs,
+                                         int ring, int launches, int64_t m, int64_t k, int64_t n, int64_t lda, void *workspace,
+                                         int64_t workspace_bytes, void *const *start_events, void *const *stop_events,
+                                         void *stream) {
+    if (a == nullptr || weights == nullptr || scales == nullptr || outs == nullptr || ring <= 0 || launches < 0) {
+        hidet_set_last_error("hidet_qmm_gemv_ring_timed: null array or empty ring");
+        return;
+    }
+    for (int i = 0; i < launches; ++i) {
+        if (start_events != nullptr && stop_events != nullptr) hidet_qmm_arm_timing(start_events[i], stop_events[i]);
+        const int r = i % ring;
+        // the operator's own entry point, called in a loop without the host interpreter between two launches; an error
+        // (last-error string set) ends the loop
+        hidet_symmetric_quant_matmul_f16_i8(a, weights[r], scales[r], outs[r], m, k, n, lda, 0, workspace, workspace_bytes, stream);
+        if (qmm::error_pending()) return;
+    }
+}
+
 HIDET_API void hidet_qmm_set_exchange_spin_limit(int limit) {
     qmm::exchange_spin_limit().store(limit < 0 ? qmm::kExchangeSpinLimit : limit, std::memory_order_relaxed);
 }

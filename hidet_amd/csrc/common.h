@@ -85,6 +85,8 @@ struct TimingSlot {
     hipEvent_t start = nullptr, stop = nullptr;
 };
 TimingSlot &timing_slot();
+// true while this thread's last-error string has not been read (it stays set)
+bool error_pending();
 
 template <typename... KArgs, typename... Args>
 inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args) {

@@ -13,6 +13,7 @@ ErrorState &error_state() {
 }  // namespace
 
 namespace qmm {
+bool error_pending() { return error_state().has_error; }
 TimingSlot &timing_slot() {
     static thread_local TimingSlot s;
     return s;

@@ -42,6 +42,7 @@ SIGNATURES = {
     'hidet_qmm_event_synchronize': (None, [_vp]),
     'hidet_qmm_event_elapsed_ms': (_f32, [_vp, _vp]),
     'hidet_qmm_arm_timing': (None, [_vp, _vp]),
+    'hidet_qmm_gemv_ring_timed': (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i64, _i64, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     'hidet_qmm_read_probe': (None, [_vp, _i64, _vp, _vp]),
     'hidet_qmm_pattern_probe': (None, [_vp, _i64, _i64, _i32, _i32, _vp, _vp]),
     'hidet_qmm_set_exchange_spin_limit': (None, [_i32]),

@@ -23,6 +23,15 @@ void hidet_qmm_event_synchronize(void *event);
 float hidet_qmm_event_elapsed_ms(void *start, void *stop);
 void hidet_qmm_arm_timing(void *start_event, void *stop_event);
 
+/* launches `launches` W8A16 matmuls (hidet_symmetric_quant_matmul_f16_i8 with parallel_k_parts = 0, one activation block a
+ * [m, k] against weights[i % ring], scales[i % ring] into outs[i % ring]) back to back from one native loop, launch i
+ * recording its own begin and end into start_events[i] / stop_events[i] (both arrays may be NULL: untimed).  What a timed
+ * pass of a benchmark needs so that the host interpreter's time per call (about as long as a decode kernel runs) does not
+ * drain the stream's queue between two launches.  An error ends the loop and is reported as usual. */
+void hidet_qmm_gemv_ring_timed(const void *a, const void *const *weights, const void *const *scales, void *const *outs, int ring,
+                               int launches, int64_t m, int64_t k, int64_t n, int64_t lda, void *workspace,
+                               int64_t workspace_bytes, void *const *start_events, void *const *stop_events, void *stream);
+
 /* ---- kernels that only read ------------------------------------------------------------------------
  * One kernel that reads `bytes` (a multiple of 32768) from src with 16-byte loads, 32 KiB contiguous per workgroup,
  * and does nothing else (sink: 4 bytes of device memory, practically never written).  Timed through the hook above it
