@@ -399,13 +399,31 @@ def main():
 
     # ---- the other benchmark configurations, one figure each (kernel duration through the timing hook, distinct weight
     # buffers per launch so that nothing is served from the last-level cache) ------------------------------------------
-    def time_kernel(fn, reps, skip):
+    # A spin kernel of about 300 us that a batch of short launches is queued behind: the host needs about as long per call
+    # as a decode kernel runs, so without it the stream's queue can run dry inside a batch and the kernels start on an
+    # idle memory system. torch's sleep kernel counts a clock whose rate is measured here once.
+    with torch.cuda.stream(stream):
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda._sleep(1000)
+        t0.record(stream)
+        torch.cuda._sleep(1000000)
+        t1.record(stream)
+    t1.synchronize()
+    blocker_cycles = int(300.0 / max(t0.elapsed_time(t1) * 1e3, 1.0) * 1000000)
+
+    def queue_blocker():
+        with torch.cuda.stream(stream):
+            torch.cuda._sleep(blocker_cycles)
+
+    def time_kernel(fn, reps, skip, short=True):
         # launches go out back to back in batches of 16, each with its own pair of events: the duration of a dispatch
         # in a busy stream, as in a decode step, not that of a kernel started on an idle chip
         pairs = [(lib.hidet_qmm_event_create(), lib.hidet_qmm_event_create()) for _ in range(16)]
         d = []
         for r0 in range(0, reps, 16):
             nb = min(16, reps - r0)
+            if short:  # decode-sized kernels; the GEMMs run far longer than the host needs per call
+                queue_blocker()
             for j in range(2):  # untimed: a batch starts behind a synchronisation, a decode step does not
                 fn(r0 + nb - 1 - j)
             for j in range(nb):
@@ -491,11 +509,11 @@ def main():
     sq = torch.cat([ss[0], ss[1]])[:12288].contiguous()
     cq = torch.empty((MP, 12288), dtype=torch.float16, device=device)
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8', ap, wq[r % 4], sq, cq, MP, K, 12288, K, 0, work,
-                                      work.numel(), sptr), 16, 4)
+                                      work.numel(), sptr), 16, 4, short=False)
     others['w8a16_prefill_m2048_k4096_n12288'] = mfma_entry(us, 2.0 * MP * K * 12288, MFMA_F16_PEAK_TFLOPS)
     # the M = 2048 prefill GEMM on K-contiguous weights (the ring's buffers read as [N, K] storage; another layout), and 32 rows
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ap, ws[r % RING].view(N, K), ss[0], cp, MP, K, N, K, K,
-                                      work, work.numel(), sptr), 16, 4)
+                                      work, work.numel(), sptr), 16, 4, short=False)
     others['w8a16_prefill_m2048_k4096_n11008_k_contiguous_weights'] = mfma_entry(us, 2.0 * MP * K * N, MFMA_F16_PEAK_TFLOPS)
     us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_f16_i8_nk', ap[:32], ws[r % RING].view(N, K), ss[0], cp[:32], 32, K, N,
                                       K, K, work, work.numel(), sptr), 32, 16)
@@ -511,7 +529,7 @@ def main():
         a4 = torch.randn((m4, K), generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
         c4 = torch.empty((m4, N), dtype=torch.bfloat16, device=device)
         us = time_kernel(lambda r: ffi.call('hidet_symmetric_quant_matmul_w4a16', a4, w4[r % 24], s4, c4, m4, K, N, K, 128, 2, 0,
-                                          work, work.numel(), sptr), 48, 24)
+                                          work, work.numel(), sptr), 48, 24, short=m4 <= 16)
         nbytes = K * N // 2 + 2 * (K // 128) * N + 2 * m4 * K + 2 * m4 * N
         others['w4a16_m{}_k4096_n11008'.format(m4)] = (hbm_entry(us, nbytes) if m4 <= 16 else
                                                       mfma_entry(us, 2.0 * m4 * K * N, MFMA_F16_PEAK_TFLOPS))
