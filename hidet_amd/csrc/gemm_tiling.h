@@ -221,6 +221,121 @@ __device__ __forceinline__ bool gemm_k_split_fixup(float4_t (&acc)[R][T], const 
     return true;
 }
 
+// ---- runs across the tiles ------------------------------------------------------------------------------------------
+//
+// When an XCD has no whole number of rounds of tiles, equal K ranges per tile leave CUs idle (22 tiles on 32 CUs) or
+// add rounds (66 thirds on 32 CUs). Here the (tile, stage) units of an XCD's region - tiles in panel order, a tile's
+// stages in order - are cut into `wgs` runs of equal length, one per workgroup, whatever the tile boundaries: a
+// workgroup computes the end of one tile, whole tiles, and the beginning of another. A bound closer than
+// kGemmStreamMinStages to a tile boundary is moved onto it, so that no piece is shorter than a pipeline's prologue.
+// A tile computed in pieces is summed by the workgroup that arrives last, in the order of the pieces
+// (gemm_stream_fixup); its pieces come from consecutive workgroups, piece p from workgroup first + p. A workgroup
+// leaves at most two pieces: the first of its run (kind 0) and, if that is a different one, the last (kind 1), which
+// gives every piece a storage slot of its own, (workgroup, kind), however many tiles there are.
+constexpr int kGemmStreamMinStages = 4;
+constexpr int kGemmStreamMinShare = 4 * kGemmStreamMinStages;  // shortest run per workgroup the planner accepts: bounds stay apart
+
+// First unit of workgroup j (0 .. wgs) of an XCD with `units` = tiles x stages units.
+__host__ __device__ __forceinline__ int gemm_stream_bound(int units, int stages, int wgs, int j) {
+    if (j <= 0) return 0;
+    if (j >= wgs) return units;
+    int raw = int((int64_t(units) * j) / wgs);
+    const int t = raw / stages, r = raw - t * stages;
+    if (r < kGemmStreamMinStages) raw = t * stages;
+    else if (stages - r < kGemmStreamMinStages) raw = (t + 1) * stages;
+    return raw;
+}
+// The workgroup whose run holds unit u.
+__host__ __device__ __forceinline__ int gemm_stream_owner(int units, int stages, int wgs, int u) {
+    int j = int((int64_t(u) * wgs) / units);  // moved bounds shift the answer by one at most
+    while (j > 0 && gemm_stream_bound(units, stages, wgs, j) > u) --j;
+    while (j + 1 < wgs && gemm_stream_bound(units, stages, wgs, j + 1) <= u) ++j;
+    return j;
+}
+
+// One piece of a workgroup's run: stages [s_begin, s_end) of region tile `local`.
+struct GemmStreamPiece {
+    int local;           // tile of the XCD's region, in panel order
+    int s_begin, s_end;
+    int part, parts;     // parts == 1: the whole tile, nothing to exchange
+    int first;           // workgroup (of the XCD) that computes piece 0
+};
+// Piece of workgroup j that lies in region tile `local` (the caller walks local from bound(j) / stages while
+// local * stages < bound(j + 1)).
+__host__ __device__ __forceinline__ GemmStreamPiece gemm_stream_piece(int units, int stages, int wgs, int j, int local) {
+    const int lo = gemm_stream_bound(units, stages, wgs, j), hi = gemm_stream_bound(units, stages, wgs, j + 1);
+    const int t0 = local * stages, t1 = t0 + stages;
+    GemmStreamPiece p;
+    p.local = local;
+    p.s_begin = (lo > t0 ? lo : t0) - t0;
+    p.s_end = (hi < t1 ? hi : t1) - t0;
+    p.part = 0;
+    p.parts = 1;
+    p.first = j;
+    if (p.s_begin != 0 || p.s_end != stages) {
+        p.first = gemm_stream_owner(units, stages, wgs, t0);
+        p.parts = gemm_stream_owner(units, stages, wgs, t1 - 1) - p.first + 1;
+        p.part = j - p.first;
+    }
+    return p;
+}
+// Storage kind of the piece workgroup j holds of region tile `local`: 0 when the tile is the first of its run.
+__host__ __device__ __forceinline__ int gemm_stream_kind(int units, int stages, int wgs, int j, int local) {
+    return gemm_stream_bound(units, stages, wgs, j) / stages == local ? 0 : 1;
+}
+
+// Fix-up of a tile computed in pieces by runs across the tiles: as gemm_k_split_fixup, with every piece in its
+// workgroup's own storage. `own` and `piece_at(p)` are the storage (THREADS * R * T * 4 floats each) of this
+// workgroup's piece and of piece p of the tile, `counter` the tile's arrival counter (zero between launches).
+template <int THREADS, int R, int T, typename PieceAt>
+__device__ __forceinline__ bool gemm_stream_fixup(float4_t (&acc)[R][T], int parts, float *__restrict__ own, PieceAt piece_at,
+                                                  uint32_t *__restrict__ counter, int *flag, uint32_t rows_valid) {
+    constexpr int kTileFloats = THREADS * R * T * 4;
+    constexpr int kAgentScope = 1 << 4;  // sc1
+    constexpr int kOutside = 0x7FFFFFF0;  // past the end of the buffer: the store is dropped, the load returns zero
+    const int lane_off = threadIdx.x * 16;
+    {
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(own, 0, kTileFloats * 4, 0x00020000);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int off = ((rows_valid >> r) & 1u) ? lane_off : kOutside;
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v_t, acc[r][t]), rsrc, off, (r * T + t) * (THREADS * 16), kAgentScope);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // every store of this lane has been acknowledged (they write through)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = (old == uint32_t(parts - 1));
+        if (*flag) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const bool last = *flag != 0;
+    __syncthreads();  // the flag is read by all before a later piece of this workgroup writes it again
+    if (!last) return false;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < parts; ++p) {
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(piece_at(p), 0, kTileFloats * 4, 0x00020000);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int off = ((rows_valid >> r) & 1u) ? lane_off : kOutside;
+            uint4v_t v[T];
+#pragma unroll
+            for (int t = 0; t < T; ++t) v[t] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, (r * T + t) * (THREADS * 16), kAgentScope);
+#pragma unroll
+            for (int t = 0; t < T; ++t) acc[r][t] += __builtin_bit_cast(float4_t, v[t]);
+        }
+    }
+    return true;
+}
+
 // Tiles XCD `xcd` owns (host-side twin of gemm_region_of_xcd).
 inline int gemm_region_tiles(const GemmTiling &t, int xcd) {
     const int xr = xcd / t.xn, xc = xcd % t.xn;

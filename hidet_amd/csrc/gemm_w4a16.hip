@@ -524,20 +524,18 @@ __device__ __forceinline__ void lds_wait_keep_newer(int4v_t (&f)[4], int4v_t (&g
                  : "n"(NEWER));
 }
 
-template <int DT>
-__global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
-    const uint16_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ w, const uint16_t *__restrict__ scales,
-    uint16_t *__restrict__ c, int m, int k, int n, int group, int tiles_m, int tiles_n, int xm, int xn, int concurrent,
-    int tail_parts, int tail_stride, float *__restrict__ partials, uint32_t *__restrict__ counters) {
+// Stages [s_begin, s_end) of output tile (tile_m, tile_n), by the whole workgroup. `split`: the tile is computed in
+// pieces and fix(acc, rows_valid) exchanges them; it returns true in the workgroup that finishes the tile.
+template <int DT, typename Fix>
+__device__ __forceinline__ void gemm_w4a16_lds_tile(const uint16_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ w,
+                                                    const uint16_t *__restrict__ scales, uint16_t *__restrict__ c, int m, int k, int n,
+                                                    int group, int tile_m, int tile_n, int s_begin, int s_end, bool split, Fix fix) {
     using Cfg = GemmW4LdsCfg;
     using T = W4G<DT>;
     extern __shared__ uint4 lds[];  // no static LDS in this kernel: every access addresses the ring from 0
-    int &s_last = *reinterpret_cast<int *>(lds + Cfg::kRingBytes / 16);
 
-    GemmWorkItem item;
-    if (!gemm_work_item(tiles_m, tiles_n, xm, xn, concurrent, tail_parts, tail_stride, &item)) return;
-    const int m0 = item.tile_m * Cfg::kBM;
-    const int n0 = item.tile_n * Cfg::kBN;
+    const int m0 = tile_m * Cfg::kBM;
+    const int n0 = tile_n * Cfg::kBN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -575,7 +573,6 @@ __global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
     const int sq_off = sq_col < n ? sq_col * 2 : kOutside;
 
     const int stages = k / kBK;
-    const int s_begin = (stages * item.part) / item.parts, s_end = (stages * (item.part + 1)) / item.parts;
 
     // A short matrix leaves most of a 256-row tile empty: a wave skips the activation loads whose 8 rows all lie past
     // the end (instruction j of wave v brings rows 64 j + 8 v .. + 7) and, if its 64 output rows do, its fragment reads
@@ -789,11 +786,11 @@ __global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // LDS must not be released with loads in flight
     __builtin_amdgcn_sched_barrier(0);
 
-    if (item.parts > 1) {
+    if (split) {
         uint32_t rows_valid = 0;  // row blocks of this wave that reach into the matrix
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb) rows_valid |= uint32_t(m0 + wm * 64 + rb * 16 < m) << rb;
-        if (!gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, &s_last, rows_valid)) return;
+        if (!fix(acc, rows_valid)) return;
     }
 
     const int col = n0 + wn * 64 + ns * 4;  // first of this lane's 4 columns
@@ -810,6 +807,51 @@ __global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
                 *reinterpret_cast<uint2 *>(c + int64_t(row) * n + col) = o;
             }
         }
+}
+
+// STREAM false: one work item per workgroup (a tile, or one of `tail_parts` equal K ranges of a tail tile). STREAM true:
+// the grid is `concurrent` workgroups per XCD and a workgroup computes its run of (tile, stage) units of the XCD's
+// region (gemm_tiling.h: runs across the tiles), piece by piece; `tail_stride` is then the stride of the per-XCD blocks
+// of tile counters, and `partials` holds two pieces per workgroup.
+template <int DT, bool STREAM>
+__global__ __launch_bounds__(512, 1) void gemm_w4a16_lds_kernel(
+    const uint16_t *__restrict__ a, int64_t lda, const uint8_t *__restrict__ w, const uint16_t *__restrict__ scales,
+    uint16_t *__restrict__ c, int m, int k, int n, int group, int tiles_m, int tiles_n, int xm, int xn, int concurrent,
+    int tail_parts, int tail_stride, float *__restrict__ partials, uint32_t *__restrict__ counters) {
+    using Cfg = GemmW4LdsCfg;
+    extern __shared__ uint4 lds[];
+    int *s_last = reinterpret_cast<int *>(lds + Cfg::kRingBytes / 16);
+    const int stages = k / kBK;
+    if constexpr (!STREAM) {
+        GemmWorkItem item;
+        if (!gemm_work_item(tiles_m, tiles_n, xm, xn, concurrent, tail_parts, tail_stride, &item)) return;
+        gemm_w4a16_lds_tile<DT>(a, lda, w, scales, c, m, k, n, group, item.tile_m, item.tile_n, (stages * item.part) / item.parts,
+                                (stages * (item.part + 1)) / item.parts, item.parts > 1, [&](auto &acc, uint32_t rows_valid) {
+                                    return gemm_k_split_fixup<Cfg::kThreads>(acc, item, partials, counters, s_last, rows_valid);
+                                });
+    } else {
+        constexpr int kTileFloats = Cfg::kBM * Cfg::kBN;
+        const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;  // workgroup b runs on XCD b % 8
+        const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, xm, xn, xcd);
+        const int units = reg.rows * reg.cols * stages;
+        if (units == 0) return;
+        const int hi = gemm_stream_bound(units, stages, concurrent, j + 1);
+        for (int local = gemm_stream_bound(units, stages, concurrent, j) / stages; local * stages < hi; ++local) {
+            const GemmStreamPiece piece = gemm_stream_piece(units, stages, concurrent, j, local);
+            int tile_m, tile_n;
+            gemm_tile_of_region(reg, local, &tile_m, &tile_n);
+            gemm_w4a16_lds_tile<DT>(a, lda, w, scales, c, m, k, n, group, tile_m, tile_n, piece.s_begin, piece.s_end, piece.parts > 1,
+                                    [&](auto &acc, uint32_t rows_valid) {
+                                        const auto piece_at = [&](int p) {
+                                            const int jp = piece.first + p;
+                                            return partials + int64_t((jp * 8 + xcd) * 2 + gemm_stream_kind(units, stages, concurrent, jp, local)) * kTileFloats;
+                                        };
+                                        return gemm_stream_fixup<Cfg::kThreads>(acc, piece.parts, piece_at(piece.part), piece_at,
+                                                                                counters + xcd * tail_stride + local, s_last, rows_valid);
+                                    });
+            __syncthreads();  // every wave is done with the rings before the next piece's loads write them
+        }
+    }
 }
 
 template <int DT>
@@ -829,8 +871,31 @@ void launch_lds(const void *a, const void *w, const void *scales, void *c, int64
         --tail.parts;
     const int64_t grid = gemm_grid_with_tail(tiling, kConcurrent, tail);
     QMM_CHECK(grid < (int64_t(1) << 31), "problem too large for one launch");
-    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w4a16_lds_kernel<DT>), Cfg::kLdsBytes);
-    launch(gemm_w4a16_lds_kernel<DT>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
+    // Runs across the tiles instead (gemm_tiling.h), one workgroup per CU, when the busiest XCD has a few tiles more than
+    // a whole number of rounds: measured against the plan above at K = 4096, N = 11008, the run plan costs about a third
+    // of a round whatever the size (a second prologue per workgroup and 128 KiB per piece through memory), so it wins
+    // where the few tail tiles would cost half a round (M = 768, 33 tiles per XCD: 123 -> 105 us; M = 1536, 65: 194 ->
+    // 187 us) and nowhere else (M = 512, 22 tiles on 32 CUs: 80 against 78 us with a third of the CUs idle; M = 1024: 129
+    // against 127 us; M = 4096: 450 against 416 us, the workgroups of a region no longer walk K in step and share less
+    // in the L2)
+    const int stages = int(k / kBK);
+    int fewest = tiling.region_tiles;
+    for (int x = 0; x < 8; ++x) fewest = std::min(fewest, gemm_region_tiles(tiling, x));
+    const int rest = tiling.region_tiles % kConcurrent;
+    const bool stream_pays = tiling.region_tiles > kConcurrent && tiling.region_tiles < 3 * kConcurrent && rest >= 1 && rest <= kConcurrent / 8;
+    const bool stream_ok = fewest > 0 && int64_t(fewest) * stages >= int64_t(kConcurrent) * kGemmStreamMinShare &&
+                           int64_t(8) * tiling.region_tiles <= kExchangeLostWord &&
+                           ws.scratch_bytes >= int64_t(8) * kConcurrent * 2 * Cfg::kBM * Cfg::kBN * 4;
+    if (stream_ok && stream_pays) {
+        allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w4a16_lds_kernel<DT, true>), Cfg::kLdsBytes);
+        launch(gemm_w4a16_lds_kernel<DT, true>, dim3(8 * kConcurrent), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
+               static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
+               static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent, 1,
+               tiling.region_tiles, reinterpret_cast<float *>(ws.scratch), ws.counters);
+        return;
+    }
+    allow_dynamic_lds(reinterpret_cast<const void *>(gemm_w4a16_lds_kernel<DT, false>), Cfg::kLdsBytes);
+    launch(gemm_w4a16_lds_kernel<DT, false>, dim3(uint32_t(grid)), dim3(Cfg::kThreads), size_t(Cfg::kLdsBytes), stream,
            static_cast<const uint16_t *>(a), lda, static_cast<const uint8_t *>(w), static_cast<const uint16_t *>(scales),
            static_cast<uint16_t *>(c), int(m), int(k), int(n), group, tiles_m, tiles_n, tiling.xm, tiling.xn, kConcurrent,
            tail.parts, tail.max_tiles, reinterpret_cast<float *>(ws.scratch), ws.counters);

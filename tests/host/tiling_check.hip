@@ -54,6 +54,62 @@ static int check(int tiles_m, int tiles_n, int concurrent, int fill, int max_par
     return 0;
 }
 
+// Runs across the tiles: every (tile, stage) of every XCD's region belongs to exactly one piece, a tile's pieces are
+// numbered 0 .. parts - 1 in stage order and come from consecutive workgroups starting at `first`, no piece is shorter
+// than kGemmStreamMinStages unless it is a whole tile's rest, and no two pieces share a storage slot (workgroup, kind).
+static int check_stream(int tiles_m, int tiles_n, int stages, int wgs) {
+    const GemmTiling t = make_gemm_tiling(tiles_m, tiles_n, wgs);
+    std::vector<int> covered(size_t(tiles_m) * tiles_n * stages, 0);
+    for (int xcd = 0; xcd < 8; ++xcd) {
+        const GemmRegion reg = gemm_region_of_xcd(tiles_m, tiles_n, t.xm, t.xn, xcd);
+        const int tiles = reg.rows * reg.cols, units = tiles * stages;
+        if (tiles == 0) continue;
+        if (int64_t(tiles) * stages < int64_t(wgs) * kGemmStreamMinShare) continue;  // the launcher does not use the plan then
+        std::vector<int> parts_of(tiles, 0), next_part(tiles, 0), next_stage(tiles, 0), first_of(tiles, -1);
+        std::vector<int> slot_used(size_t(wgs) * 2, 0);
+        int prev = 0;
+        for (int j = 0; j < wgs; ++j) {
+            const int lo = gemm_stream_bound(units, stages, wgs, j), hi = gemm_stream_bound(units, stages, wgs, j + 1);
+            if (lo != prev || hi <= lo) return std::printf("stream %dx%d s%d: workgroup %d of XCD %d runs [%d, %d) after %d\n", tiles_m, tiles_n, stages, j, xcd, lo, hi, prev), 1;
+            prev = hi;
+            for (int u = lo; u < hi; ++u)
+                if (gemm_stream_owner(units, stages, wgs, u) != j) return std::printf("stream %dx%d s%d: owner of unit %d is not %d\n", tiles_m, tiles_n, stages, u, j), 1;
+            int pieces = 0;
+            for (int local = lo / stages; local * stages < hi; ++local) {
+                const GemmStreamPiece p = gemm_stream_piece(units, stages, wgs, j, local);
+                if (p.local != local || p.s_begin < 0 || p.s_end > stages || p.s_begin >= p.s_end || p.s_begin != next_stage[local])
+                    return std::printf("stream %dx%d s%d: workgroup %d tile %d stages [%d, %d), expected from %d\n", tiles_m, tiles_n, stages, j, local, p.s_begin, p.s_end, next_stage[local]), 1;
+                next_stage[local] = p.s_end;
+                if (p.part != next_part[local] || (parts_of[local] != 0 && parts_of[local] != p.parts) || p.part >= p.parts ||
+                    (first_of[local] >= 0 && first_of[local] != p.first) || p.first + p.part != j)
+                    return std::printf("stream %dx%d s%d: workgroup %d tile %d part %d/%d first %d\n", tiles_m, tiles_n, stages, j, local, p.part, p.parts, p.first), 1;
+                parts_of[local] = p.parts;
+                first_of[local] = p.first;
+                ++next_part[local];
+                if (p.parts > 1) {
+                    if (p.s_end - p.s_begin < kGemmStreamMinStages) return std::printf("stream %dx%d s%d: piece of %d stages\n", tiles_m, tiles_n, stages, p.s_end - p.s_begin), 1;
+                    const int kind = gemm_stream_kind(units, stages, wgs, j, local);
+                    if (slot_used[j * 2 + kind]++) return std::printf("stream %dx%d s%d: workgroup %d uses storage %d twice\n", tiles_m, tiles_n, stages, j, kind), 1;
+                    ++pieces;
+                } else if (p.s_begin != 0 || p.s_end != stages) {
+                    return std::printf("stream %dx%d s%d: a lone piece [%d, %d)\n", tiles_m, tiles_n, stages, p.s_begin, p.s_end), 1;
+                }
+                int tm, tn;
+                if (!gemm_tile_of_region(reg, local, &tm, &tn)) return std::printf("stream %dx%d: tile %d outside the region\n", tiles_m, tiles_n, local), 1;
+                for (int st = p.s_begin; st < p.s_end; ++st) ++covered[(size_t(tm) * tiles_n + tn) * stages + st];
+            }
+            if (pieces > 2) return std::printf("stream %dx%d s%d: workgroup %d leaves %d pieces\n", tiles_m, tiles_n, stages, j, pieces), 1;
+        }
+        if (prev != units) return std::printf("stream %dx%d s%d: runs end at %d of %d\n", tiles_m, tiles_n, stages, prev, units), 1;
+        for (int local = 0; local < tiles; ++local)
+            if (next_stage[local] != stages || next_part[local] != parts_of[local])
+                return std::printf("stream %dx%d s%d: tile %d ends at stage %d, %d of %d parts\n", tiles_m, tiles_n, stages, local, next_stage[local], next_part[local], parts_of[local]), 1;
+    }
+    for (int seen : covered)
+        if (seen > 1) return std::printf("stream %dx%d s%d: a stage of a tile belongs to two XCDs\n", tiles_m, tiles_n, stages), 1;
+    return 0;
+}
+
 // Bandwidth-bound kernels: the (tile, 32-row step) units of a launch are dealt to workgroups and waves in one flat run
 // each. Every unit must belong to exactly one wave, a workgroup's run may touch two tiles at most, every tile has one
 // collector (the workgroup with its last unit) that fetches exactly the slots of the workgroups before it in the tile,
@@ -194,6 +250,13 @@ int main() {
                 if (check(tm, tn, c[0], 2, c[2], 3)) return 1;
                 n += 5;
             }
+    for (int stages : {16, 17, 43, 64, 172, 448})
+        for (int tm = 1; tm <= 40; tm += (tm < 10 ? 1 : 5))
+            for (int tn = 1; tn <= 130; tn += (tn < 50 ? 3 : 9))
+                for (int wgs : {32, 64}) {
+                    if (check_stream(tm, tn, stages, wgs)) return 1;
+                    ++n;
+                }
     std::printf("ok %lld launches\n", n);
     return 0;
 }

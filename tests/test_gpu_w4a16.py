@@ -143,6 +143,42 @@ def test_k_split_is_deterministic():
         assert np.array_equal(host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g)), first)
 
 
+@pytest.mark.parametrize('m,k,n', [(768, 2048, 11008), (1536, 1024, 11008), (700, 4096, 11008)])
+def test_runs_across_the_tiles(m, k, n):
+    """33 (65) tiles of 256 x 128 on the busiest XCD, one (one) more than whole rounds of 32 workgroups: the launcher deals
+    every XCD's (tile, stage) units to 32 workgroups in equal runs, and tiles computed in pieces are summed by the last
+    workgroup to arrive. Small integers and power-of-two scales: every sum is exact whatever the pieces, so the
+    result must equal integer arithmetic bit for bit; and twice the same."""
+    announce('w4a16 runs across tiles', m, k, n)
+    rng = np.random.default_rng(m + k)
+    a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    q = rng.integers(-8, 8, (k, n)).astype(np.int8)
+    scales = (2.0 ** rng.integers(-3, 1, (k // 128, n))).astype(np.float32)
+    ta, tp, ts = dev(a, torch.bfloat16), dev(O.pack_int4(q)), dev(scales, torch.bfloat16)
+    got = host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, 128))
+    rows = np.unique(np.concatenate([np.arange(0, m, 37), [255, 256, 511, 512, m - 1]]))
+    want = np.zeros((len(rows), n))
+    for g in range(k // 128):
+        want += (a[rows, g * 128:(g + 1) * 128].astype(np.int64) @ q[g * 128:(g + 1) * 128].astype(np.int64)) * scales[g]
+    assert np.array_equal(got[rows], O.to_bf16(want.astype(np.float32)))
+    assert np.array_equal(host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, 128)), got)
+    # against the rows computed one 16-row batch at a time by the bandwidth-bound kernel (no tiles, no pieces)
+    idx = torch.from_numpy(rows[:16]).cuda()
+    assert np.array_equal(host(quant.symmetric_quant_matmul_w4a16(ta[idx].contiguous(), tp, ts, 128)), got[rows[:16]])
+
+
+def test_runs_across_the_tiles_random_operands():
+    m, k, n, g = 768, 2048, 11008, 128
+    announce('w4a16 runs across tiles, random', m, k, n)
+    a, packed, scales, ta, tp, ts = _case(5, m, k, n, g, 'bfloat16')
+    got = host(quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g))
+    rows = np.array([0, 100, 255, 256, 300, 511, 512, 640, 767])
+    ref = O.w4a16_matmul(a[rows], packed, scales, g, 'bfloat16')
+    err = O.max_rel_err(got[rows], ref)
+    print('max_rel_err', err)
+    assert err <= 8e-3
+
+
 def test_full_size_prefill_rows_sample():
     m, k, n, g = 512, 4096, 11008, 128
     announce('w4a16 full size', m, k, n)
