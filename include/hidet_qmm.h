@@ -31,7 +31,9 @@
  *       the same with more rows, hidet_matmul_f8, hidet_matmul_f8_scaled, the _nk matmuls
  *                                         scratch: 64 KiB per tile computed in K ranges times the ranges (optional: with
  *                                         less, fewer or no tiles are split; hidet_qmm_min_workspace_bytes() serves
- *                                         every shape).
+ *                                         every shape); hidet_symmetric_quant_matmul_w4a16 with a few hundred to a few
+ *                                         thousand rows: 64 MiB for its plan of equal runs of work per workgroup
+ *                                         (optional: with less it computes whole tiles and equal K ranges).
  *     hidet_qmm_workspace_bytes_for_scratch(s) returns the smallest workspace whose scratch part holds s bytes.
  *
  * All tensors are dense row-major.  No function allocates device memory; none but hidet_qmm_exchange_status synchronises.
