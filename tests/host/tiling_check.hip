@@ -227,7 +227,7 @@ int main() {
     for (long long ws : {0LL, 1024LL, 65536LL, 65536LL + 8192, 1LL << 20, 16LL << 20, (16LL << 20) + 65536, 64LL << 20, 96LL << 20})
         for (long long k : {32LL, 96LL, 128LL, 1000LL, 4096LL, 11008LL, 16384LL, 28672LL})
             for (long long nc : {2LL, 16LL, 256LL, 272LL, 4096LL, 11008LL, 12288LL, 128256LL})
-                for (int rows : {1, 8, 16})
+                for (int rows : {1, 2, 8, 16})
                     for (int hint : {0, 1, 3, 8, 64}) {
                         if (check_skinny(k, nc, hint, rows, ws, true, 256)) return 1;
                         if (check_skinny(k, nc, hint, rows, ws, false, 256)) return 1;
