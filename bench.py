@@ -123,6 +123,9 @@ def main():
                          'at 4096 x 11008, W8A16 M = 16 at 4096 x 4096, the headline GEMV for comparison), over distinct weight buffers')
     ap.add_argument('--skip-two-chains', action='store_true',
                     help='leave out the two-stream graph: under a kernel trace its overlapping launches would blur the GEMV kernel\'s average duration')
+    ap.add_argument('--skip-exchange-probe', action='store_true',
+                    help='leave out the GEMV passes with a poll limit of zero (launches that never wait for the exchange): under a '
+                         'kernel trace they cannot be told from the measured launches and would pull the kernel\'s average down')
     ap.add_argument('--data-dependence', action='store_true',
                     help='time the two GEMM kernels on all-zero operands and on the benchmark operands: the instruction '
                          'stream is identical, the difference is the clock the chip sustains under its power limit')
@@ -279,21 +282,38 @@ def main():
     ev_array = ctypes.c_void_p * (LAPS * RING)
     w_ptrs, s_ptrs, o_ptrs = (ptr_array(*[t.data_ptr() for t in ts]) for ts in (ws, ss, outs))
     e0s, e1s = ev_array(*[e[0] for e in evs]), ev_array(*[e[1] for e in evs])
-    durs = []
-    for rep in range(5):
-        # one native loop per pass: an untimed lap (the pass starts behind a synchronisation, the timed region does not),
-        # then the timed launches. Issued from Python one call at a time, a launch costs the host about as long as the
-        # kernel runs, and on a slow host the stream's queue runs dry in the later laps of a pass: the kernels then start
-        # on an idle memory system and take 0.5-1.5 us longer (seen as a mean that grows from lap to lap)
-        ffi.call('hidet_qmm_gemv_ring_timed', a, w_ptrs, s_ptrs, o_ptrs, RING, RING, 1, K, N, K, work, work.numel(), None, None, sptr)
-        ffi.call('hidet_qmm_gemv_ring_timed', a, w_ptrs, s_ptrs, o_ptrs, RING, LAPS * RING, 1, K, N, K, work, work.numel(), e0s, e1s, sptr)
+    def native_passes(passes):
+        durs = []
+        for rep in range(passes):
+            # one native loop per pass: an untimed lap (the pass starts behind a synchronisation, the timed region does not),
+            # then the timed launches. Issued from Python one call at a time, a launch costs the host about as long as the
+            # kernel runs, and on a slow host the stream's queue runs dry in the later laps of a pass: the kernels then start
+            # on an idle memory system and take 0.5-1.5 us longer (seen as a mean that grows from lap to lap)
+            ffi.call('hidet_qmm_gemv_ring_timed', a, w_ptrs, s_ptrs, o_ptrs, RING, RING, 1, K, N, K, work, work.numel(), None, None, sptr)
+            ffi.call('hidet_qmm_gemv_ring_timed', a, w_ptrs, s_ptrs, o_ptrs, RING, LAPS * RING, 1, K, N, K, work, work.numel(), e0s, e1s, sptr)
+            stream.synchronize()
+            durs.extend(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3 for e0, e1 in evs)
+        return np.array(durs[LAPS * RING:])  # first pass warms the instruction cache
+
+    durs = native_passes(5)
+    kernel_us = float(durs.mean())
+    # What waiting for the exchange costs: the same passes with the collectors' poll limit at zero - they read the mailbox
+    # once and give up (outputs NaN, a flag in the workspace), so no launch waits for a partial tile. Afterwards the limit
+    # goes back to its default, the workspace is put back in order, and a launch must give the parity result again.
+    no_wait_us = None
+    if not args.skip_exchange_probe:
+        lib.hidet_qmm_set_exchange_spin_limit(0)
+        no_wait_us = float(native_passes(3).mean())
+        lib.hidet_qmm_set_exchange_spin_limit(-1)
+        gave_up = lib.hidet_qmm_exchange_status(work.data_ptr(), work.numel(), sptr)
+        lib.hidet_qmm_exchange_reset(work.data_ptr(), work.numel(), sptr)
+        launch(3, sptr)
         stream.synchronize()
-        durs.extend(lib.hidet_qmm_event_elapsed_ms(e0, e1) * 1e3 for e0, e1 in evs)
+        if gave_up != 1 or O.max_rel_err(outs[3].cpu().numpy(), ref) != parity:
+            raise SystemExit('bench.py: the exchange did not recover after the run without waiting')
     for e0, e1 in evs:
         lib.hidet_qmm_event_destroy(e0)
         lib.hidet_qmm_event_destroy(e1)
-    durs = np.array(durs[LAPS * RING:])  # first pass warms the instruction cache
-    kernel_us = float(durs.mean())
     # where the slow launches are: by weight buffer (physical placement of a 45 MB buffer), by position in a pass
     # (a pass starts behind one untimed lap), by pass
     by_launch = durs.reshape(-1, LAPS, RING)
@@ -504,6 +524,11 @@ def main():
                                       ('same_bytes_per_wave_contiguous_256_workgroups', 256, 1)):
         us = time_kernel(lambda r: ffi.call('hidet_qmm_pattern_probe', ws[r % RING], K, N, groups, contiguous, sink, sptr), 64, 16)
         read_probe[label + '_45MB'] = hbm_entry(us, K * N)
+    # the GEMV's grid (256 workgroups of 512 threads) with 8 KiB to read in all: what lies between a launch's begin and end
+    # events before the matrix moves
+    us = time_kernel(lambda r: ffi.call('hidet_qmm_pattern_probe', ws[r % RING], 32, 256, 256, 0, sink, sptr), 64, 16)
+    read_probe['launch_of_the_gemv_grid_reading_8_KiB_us'] = round(us, 2)
+    read_probe['gemv_with_a_poll_limit_of_zero_us'] = None if no_wait_us is None else round(no_wait_us, 3)
     # W8A16 prefill, attention QKV shape [2048, 4096] x [4096, 12288]
     wq = [torch.randint(-127, 128, (K, 12288), device=device, dtype=torch.int8) for _ in range(4)]
     sq = torch.cat([ss[0], ss[1]])[:12288].contiguous()
