@@ -212,5 +212,9 @@ __device__ __forceinline__ _Float16 scaled_biased_f16(float acc, float scale, fl
     const _Float16 product = _Float16(acc * scale);
     return _Float16(float(product) + bias);
 }
+// The bfloat16 form (bits): the matmul's bfloat16 result, then the add rounded to bfloat16 again.
+__device__ __forceinline__ uint16_t biased_bf16_bits(float acc, float bias) {
+    return f32_to_bf16_bits(bf16_bits_to_f32(f32_to_bf16_bits(acc)) + bias);
+}
 
 }  // namespace qmm

@@ -20,6 +20,11 @@ __device__ __forceinline__ int skinny_red_chunk(int c) { return (c & ~3) | ((c ^
 
 inline size_t skinny_lds_bytes(int m, int waves) { return size_t(waves) * m * kSkinnyRedStride * sizeof(float); }
 
+// Output type of a bfloat16 kernel that adds a bias vector (bfloat16 bits) in its epilogue; plain bfloat16 bits are uint16_t.
+struct bf16_biased_t {
+    uint16_t bits;
+};
+
 template <typename OutT>
 __device__ __forceinline__ OutT skinny_to_out(float v);
 template <>
@@ -228,8 +233,8 @@ __host__ __device__ __forceinline__ bool skinny_column_layout(int m, int others,
     return (rows <= 4 && others <= 4) || (rows <= 2 && others <= 8) || (rows <= 1 && others <= 16);
 }
 
-// Column factors of the output, c = sum * scale[n] + bias[n]: float16 vectors of n elements, either may be null (scale
-// 1, bias 0). The tail fetches them while its reads of the mailbox are under way, not earlier: a load issued between the
+// Column factors of the output, c = sum * scale[n] + bias[n]: vectors of n elements of the output's 16-bit type (declared
+// float16 here; the bfloat16 kernels pass bfloat16 bits through the same pointers), either may be null (scale 1, bias 0). The tail fetches them while its reads of the mailbox are under way, not earlier: a load issued between the
 // weight loads would have to come back before the weights issued after it.
 struct SkinnyScale {
     const _Float16 *scale = nullptr, *bias = nullptr;
@@ -313,9 +318,12 @@ struct SkinnyTail {
         return r;
     }
     // one output element: float16 outputs take the column factor and the bias (two roundings, see scaled_biased_f16);
-    // bfloat16 outputs have neither (the int4 kernel folds its group scales in before)
+    // bfloat16 outputs have neither (the int4 kernel folds its group scales in before) unless the kernel asks for the bias
+    // with the output type bf16_biased_t: the same two roundings then. (A type of its own, so that the calls without a
+    // bias keep the shorter epilogue: every instruction behind the last weight delays the kernel's end.)
     __device__ __forceinline__ OutT finish(float sum, int e) const {
         if constexpr (std::is_same<OutT, _Float16>::value) return scaled_biased_f16(sum, scale[e], bias[e]);
+        else if constexpr (std::is_same<OutT, bf16_biased_t>::value) return bf16_biased_t{biased_bf16_bits(sum, bias[e])};
         else return skinny_to_out<OutT>(sum);
     }
     __device__ __forceinline__ void store(int row, const Vals &x) const {
@@ -365,8 +373,11 @@ struct SkinnyTail {
     __device__ __forceinline__ void use_factors() {
 #pragma unroll
         for (int e = 0; e < CW; ++e) {
-            scale[e] = factors.scale != nullptr ? f16_bits_to_f32(uint16_t(scale_bits[e >> 1] >> (16 * (e & 1)))) : 1.0f;
-            bias[e] = factors.bias != nullptr ? f16_bits_to_f32(uint16_t(bias_bits[e >> 1] >> (16 * (e & 1)))) : -0.0f;
+            // the vectors have the output's type: float16, or bfloat16 bits
+            const uint16_t sb = uint16_t(scale_bits[e >> 1] >> (16 * (e & 1))), bb = uint16_t(bias_bits[e >> 1] >> (16 * (e & 1)));
+            constexpr bool kHalf16 = std::is_same<OutT, _Float16>::value;
+            scale[e] = factors.scale != nullptr ? (kHalf16 ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb)) : 1.0f;
+            bias[e] = factors.bias != nullptr ? (kHalf16 ? f16_bits_to_f32(bb) : bf16_bits_to_f32(bb)) : -0.0f;
         }
     }
 

@@ -24,13 +24,13 @@ constexpr int kDepth = 2;          // 32-row steps fetched together
 // workgroups, non-temporal loads with no condition around them - rows past the wave's range lie outside the buffer and
 // read as zero bytes, which are code 0 - and the exchange of skinny_tails. A step is 32 rows and the group size a
 // multiple of 32, so a step never straddles two groups.
-template <int DT, bool ALIGNED_A>
+template <int DT, bool ALIGNED_A, bool BIAS>
 __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(int ksteps, uint32_t ksteps_magic, int per_group, int longer, int splits, uint32_t splits_magic,
                                                                         const uint8_t *__restrict__ w, const uint16_t *__restrict__ a,
                                                                         int64_t lda, int m, int k, int n, int group,
                                                                         SkinnyPlanRest plan_rest, const uint16_t *__restrict__ scales,
-                                                                        uint16_t *__restrict__ c, float *__restrict__ mailbox,
-                                                                        uint32_t *__restrict__ lost_flag) {
+                                                                        const uint16_t *__restrict__ bias, uint16_t *__restrict__ c,
+                                                                        float *__restrict__ mailbox, uint32_t *__restrict__ lost_flag) {
     using T = W4Traits<DT>;
     extern __shared__ float red[];
 
@@ -163,11 +163,15 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(int kst
         }
         skinny_stash(total, m, wave, red);
     }
-    const SkinnyScale no_scale;  // ones and no bias: the group scales are already in the totals
+    // no column factor: the group scales are already in the totals; BIAS: the bias (of the output's type) is added to the
+    // rounded result, as a matmul followed by an add would. Without one the kernels are the ones that never knew of it.
+    const SkinnyScale no_scale = {nullptr, BIAS ? reinterpret_cast<const _Float16 *>(bias) : nullptr};
     // (worked out here, not inside the loop: there it was measured to cost the loop more than it saves the tail)
     const SkinnyRoles roles = skinny_roles_of(plan, wk, grp, kSkinnyWaves);
-    if (DT == HIDET_QMM_F16)
+    if constexpr (DT == HIDET_QMM_F16)
         skinny_tails<_Float16, kSkinnyWaves>(plan, wk, roles, m, n, no_scale, reinterpret_cast<_Float16 *>(c), mailbox, lost_flag, red);
+    else if constexpr (BIAS)
+        skinny_tails<bf16_biased_t, kSkinnyWaves>(plan, wk, roles, m, n, no_scale, reinterpret_cast<bf16_biased_t *>(c), mailbox, lost_flag, red);
     else
         skinny_tails<uint16_t, kSkinnyWaves>(plan, wk, roles, m, n, no_scale, c, mailbox, lost_flag, red);
 }
@@ -176,7 +180,8 @@ __global__ __launch_bounds__(64 * kSkinnyWaves) void skinny_w4a16_kernel(int kst
 template <int DT>
 __global__ __launch_bounds__(256) void naive_w4a16_kernel(const uint16_t *__restrict__ a, int64_t lda,
                                                           const uint8_t *__restrict__ w, const uint16_t *__restrict__ scales,
-                                                          uint16_t *__restrict__ c, int64_t m, int64_t k, int64_t n, int group) {
+                                                          const uint16_t *__restrict__ bias, uint16_t *__restrict__ c, int64_t m,
+                                                          int64_t k, int64_t n, int group) {
     using T = W4Traits<DT>;
     const int64_t o = int64_t(blockIdx.x) * 256 + threadIdx.x;
     if (o >= m * n) return;
@@ -191,8 +196,9 @@ __global__ __launch_bounds__(256) void naive_w4a16_kernel(const uint16_t *__rest
         }
         total += acc * T::to_f32(scales[(g0 / group) * n + j]);
     }
-    if (DT == HIDET_QMM_F16) c[o] = f32_to_f16_bits(total);
-    else c[o] = f32_to_bf16_bits(total);
+    const float b = bias != nullptr ? T::to_f32(bias[j]) : -0.0f;  // -0.0 changes nothing, not even the sign of a zero
+    if (DT == HIDET_QMM_F16) c[o] = __builtin_bit_cast(uint16_t, scaled_biased_f16(total, 1.0f, b));
+    else c[o] = biased_bf16_bits(total, b);
 }
 
 }  // namespace
@@ -201,18 +207,19 @@ bool skinny_w4a16_fast(const void *w, const void *scales, int64_t k, int64_t n, 
     return (n % 16 == 0) && n < (int64_t(1) << 30) && (group % 32 == 0) && aligned(w, 8) && aligned(scales, 16) && k > 0;
 }
 
-void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k, int64_t n,
+void skinny_w4a16_launch(const void *a, const void *w, const void *scales, const void *bias, void *c, int64_t m, int64_t k, int64_t n,
                          int64_t lda, int group, int dtype, int parallel_k_parts, void *workspace, int64_t workspace_bytes,
                          hipStream_t stream) {
     const uint16_t *ap0 = static_cast<const uint16_t *>(a);
+    const uint16_t *bp = static_cast<const uint16_t *>(bias);
     const uint8_t *wp = static_cast<const uint8_t *>(w);
     const uint16_t *sp = static_cast<const uint16_t *>(scales);
     uint16_t *cp0 = static_cast<uint16_t *>(c);
-    if (!skinny_w4a16_fast(w, scales, k, n, group)) {
+    if (!skinny_w4a16_fast(w, scales, k, n, group) || !aligned(bias, 8)) {  // 8-byte bias loads
         if (dtype == HIDET_QMM_F16)
-            launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
+            launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, bp, cp0, m, k, n, group);
         else
-            launch(naive_w4a16_kernel<HIDET_QMM_BF16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
+            launch(naive_w4a16_kernel<HIDET_QMM_BF16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, bp, cp0, m, k, n, group);
         return;
     }
     const Workspace ws = split_workspace(workspace, workspace_bytes);
@@ -221,9 +228,9 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
     if ((cdiv(cdiv(skinny_units(plan), plan.groups), kSkinnyWaves) * 32 + 64) * (n / 2) >= (int64_t(1) << 31) - (1 << 20) ||
         (k / group) * n * 2 >= (int64_t(1) << 31) - (1 << 20)) {
         if (dtype == HIDET_QMM_F16)
-            launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
+            launch(naive_w4a16_kernel<HIDET_QMM_F16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, bp, cp0, m, k, n, group);
         else
-            launch(naive_w4a16_kernel<HIDET_QMM_BF16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, cp0, m, k, n, group);
+            launch(naive_w4a16_kernel<HIDET_QMM_BF16>, dim3(cdiv(m * n, 256)), dim3(256), 0, stream, ap0, lda, wp, sp, bp, cp0, m, k, n, group);
         return;
     }
     // 16-byte activation loads through a buffer descriptor: aligned rows, offsets below 2^31
@@ -235,15 +242,25 @@ void skinny_w4a16_launch(const void *a, const void *w, const void *scales, void 
         auto go = [&](auto kern) {
             if (shmem > 65536) allow_dynamic_lds(reinterpret_cast<const void *>(kern), int(skinny_lds_bytes(16, kSkinnyWaves)));  // the most any m needs
             launch(kern, dim3(skinny_grid(plan)), dim3(64 * kSkinnyWaves), shmem, stream, plan.ksteps, plan.ksteps_magic, plan.per_group, plan.longer, plan.splits, plan.splits_magic,
-                   wp, ap0 + m0 * lda, lda, mt, int(k), int(n), group, static_cast<SkinnyPlanRest>(plan), sp, cp0 + m0 * n, ws.mailbox,
+                   wp, ap0 + m0 * lda, lda, mt, int(k), int(n), group, static_cast<SkinnyPlanRest>(plan), sp, bp, cp0 + m0 * n, ws.mailbox,
                    lost_flag);
         };
         if (dtype == HIDET_QMM_F16) {
-            if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, true>);
-            else go(skinny_w4a16_kernel<HIDET_QMM_F16, false>);
+            if (bias != nullptr) {
+                if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, true, true>);
+                else go(skinny_w4a16_kernel<HIDET_QMM_F16, false, true>);
+            } else {
+                if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_F16, true, false>);
+                else go(skinny_w4a16_kernel<HIDET_QMM_F16, false, false>);
+            }
         } else {
-            if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_BF16, true>);
-            else go(skinny_w4a16_kernel<HIDET_QMM_BF16, false>);
+            if (bias != nullptr) {
+                if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_BF16, true, true>);
+                else go(skinny_w4a16_kernel<HIDET_QMM_BF16, false, true>);
+            } else {
+                if (aligned_a) go(skinny_w4a16_kernel<HIDET_QMM_BF16, true, false>);
+                else go(skinny_w4a16_kernel<HIDET_QMM_BF16, false, false>);
+            }
         }
     }
 }

@@ -56,6 +56,7 @@ SIGNATURES = {
     'hidet_symmetric_quant_matmul_f16_i8_nk': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _i64, _vp]),
     'hidet_group_quantize_int4': (None, [_vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
     'hidet_symmetric_quant_matmul_w4a16': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
+    'hidet_symmetric_quant_matmul_w4a16_bias': (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     'hidet_symmetric_quant_matmul_w4a16_nk': (None, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _vp]),
     'hidet_fp8_quantize_per_tensor': (None, [_vp, _vp, _vp, _i64, _i32, _vp, _i64, _vp]),
     'hidet_matmul_f8': (None, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _i64, _vp]),

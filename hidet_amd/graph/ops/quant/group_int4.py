@@ -2,7 +2,7 @@
 the reference's own: signed int4 with max 7 (python/hidet/ir/dtypes/integer_subbyte.py:49), two codes per
 byte along the innermost axis, low nibble first (python/hidet/transforms/lower_integer_subbyte.py:103-113),
 scales shaped [K / group, N] (tests/cute_kernel/quantized_linear.py:692-699)."""
-from typing import List, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -69,22 +69,35 @@ class SymmetricQuantizedMatmulW4A16Task(Task):
                          outputs=[TensorSpec('c', a.dtype, tuple(a.shape[:-1]) + (n,))], attrs={'group_size': group_size})
 
 
+def _check_bias(bias: torch.Tensor, n: int, dtype: torch.dtype) -> torch.Tensor:
+    if bias.dtype != dtype or bias.dim() != 1 or bias.shape[0] != n:
+        raise ValueError('bias must be a {} vector of {} elements, got {} {}'.format(dtype, n, bias.dtype, list(bias.shape)))
+    return bias.contiguous()
+
+
 class SymmetricQuantizedMatmulW4A16Op(Operator):
-    def __init__(self, a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, group_size: int):
+    def __init__(self, a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, group_size: int, bias: Optional[torch.Tensor] = None):
         task = SymmetricQuantizedMatmulW4A16Task(input_like(a, 'a'), input_like(packed, 'b'), input_like(scales, 'scale'), group_size)
+        if bias is not None:
+            _check_bias(bias, packed.shape[1] * 2, a.dtype)
+        self.bias = bias
         super().__init__(inputs=[a, packed, scales], attributes={'group_size': group_size}, task=task)
 
     def run(self) -> List[torch.Tensor]:
         a, packed, scales = self.inputs
-        return [_run_w4a16(a, packed, scales, self.attrs['group_size'])]
+        return [_run_w4a16(a, packed, scales, self.attrs['group_size'], self.bias)]
 
 
 _VALIDATED = set()  # operand signatures that have passed the task's checks once
 
 
-def _run_w4a16(a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, group_size: int) -> torch.Tensor:
+def _run_w4a16(a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, group_size: int,
+               bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     ffi.require_gpu(a, packed, scales)
     k, n = packed.shape[0], packed.shape[1] * 2
+    if bias is not None:
+        ffi.require_gpu(bias)
+        bias = _check_bias(bias, n, a.dtype)
     a2 = a.reshape(-1, k)
     if a2.stride(-1) != 1 or (a2.shape[0] > 1 and a2.stride(0) < k):
         a2 = a2.contiguous()
@@ -92,19 +105,27 @@ def _run_w4a16(a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, grou
     lda = a2.stride(0) if m > 1 else k
     c = torch.empty((m, n), dtype=a.dtype, device=a.device)
     ws = ffi.workspace(a.device)
-    ffi.call('hidet_symmetric_quant_matmul_w4a16', a2, packed.contiguous(), scales.contiguous(), c, m, k, n, lda,
-             group_size, ffi.DTYPE_CODE[a.dtype], 0, ws, ws.numel(), ffi.current_stream(a.device))
+    if bias is None:
+        ffi.call('hidet_symmetric_quant_matmul_w4a16', a2, packed.contiguous(), scales.contiguous(), c, m, k, n, lda,
+                 group_size, ffi.DTYPE_CODE[a.dtype], 0, ws, ws.numel(), ffi.current_stream(a.device))
+    else:
+        ffi.call('hidet_symmetric_quant_matmul_w4a16_bias', a2, packed.contiguous(), scales.contiguous(), bias, c, m, k, n, lda,
+                 group_size, ffi.DTYPE_CODE[a.dtype], 0, ws, ws.numel(), ffi.current_stream(a.device))
     return c.reshape(tuple(a.shape[:-1]) + (n,))
 
 
-def symmetric_quant_matmul_w4a16(a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, group_size: int = 128) -> torch.Tensor:
-    """c[..., M, N] = a @ dequant(packed, scales) with fp32 accumulation; a, scales and c share bfloat16 or float16."""
-    signature = (a.shape, a.dtype, packed.shape, packed.dtype, scales.shape, scales.dtype, group_size)
+def symmetric_quant_matmul_w4a16(a: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor, group_size: int = 128,
+                                 bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """c[..., M, N] = a @ dequant(packed, scales) with fp32 accumulation; a, scales and c share bfloat16 or float16.
+    `bias` ([N], the same type) is added to the rounded result: the bits of the matmul followed by an add, as for the int8
+    operator."""
+    signature = (a.shape, a.dtype, packed.shape, packed.dtype, scales.shape, scales.dtype, group_size,
+                 None if bias is None else (bias.shape, bias.dtype))
     if signature in _VALIDATED:  # checked before: skip building the operator and task records (host time of a decode call)
-        return _run_w4a16(a, packed, scales, group_size)
+        return _run_w4a16(a, packed, scales, group_size, bias)
     if len(a.shape) < 2 or len(packed.shape) < 2:
         raise ValueError('a and b must have at least 2 dimensions, got shape {} and {}'.format(list(a.shape), list(packed.shape)))
-    out = SymmetricQuantizedMatmulW4A16Op(a, packed, scales, group_size).outputs[0]
+    out = SymmetricQuantizedMatmulW4A16Op(a, packed, scales, group_size, bias).outputs[0]
     _VALIDATED.add(signature)
     return out
 

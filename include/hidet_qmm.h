@@ -24,7 +24,7 @@
  *     scratch = workspace_bytes - 65536 - mailbox.  What each entry point needs of it:
  *       hidet_symmetric_quantize          scratch >= 4 * outer * inner bytes (an error otherwise);
  *       hidet_fp8_quantize_per_tensor     scratch >= 4 bytes (an error otherwise);
- *       hidet_symmetric_quant_matmul_f16_i8[_bias], hidet_symmetric_quant_matmul_w4a16 with up to 16 rows
+ *       hidet_symmetric_quant_matmul_f16_i8[_bias], hidet_symmetric_quant_matmul_w4a16[_bias] with up to 16 rows
  *                                         mailbox >= 1024 * min(m, 16) bytes per workgroup of the K split, at most 256
  *                                         workgroups unless parallel_k_parts asks for more (4 MiB serve every automatic
  *                                         plan); with less the kernels use fewer workgroups, never an error;
@@ -169,6 +169,12 @@ void hidet_group_quantize_int4(const void *w, void *packed, void *scales, int64_
 void hidet_symmetric_quant_matmul_w4a16(const void *a, const void *w, const void *scales, void *c, int64_t m, int64_t k,
                                         int64_t n, int64_t lda, int group_size, int dtype, int parallel_k_parts,
                                         void *workspace, int64_t workspace_bytes, void *stream);
+/* The same with bias[n] (of `dtype`, not NULL) added to the rounded result, c = dtype(dtype(sum) + bias): the bits of
+ * the matmul followed by an add, as for the int8 operator (hidet_symmetric_quant_matmul_f16_i8_bias). Up to 32 rows the
+ * add rides in the kernel's epilogue; above, a short element-wise pass follows the GEMM. */
+void hidet_symmetric_quant_matmul_w4a16_bias(const void *a, const void *w, const void *scales, const void *bias, void *c,
+                                             int64_t m, int64_t k, int64_t n, int64_t lda, int group_size, int dtype,
+                                             int parallel_k_parts, void *workspace, int64_t workspace_bytes, void *stream);
 /* The same operator on weights repacked for decode: w_nk is uint8 [n, k/2] with row stride ldw bytes, row n holding
  * the k codes of output column n; inside every 32-bit word (8 consecutive k) nibble i is code 2i for i < 4 and code
  * 2(i-4)+1 for i >= 4 (hidet_amd.graph.ops.quant.to_decode_layout_int4 repacks). scales stay [k/group, n]. No

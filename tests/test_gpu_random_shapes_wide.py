@@ -90,11 +90,16 @@ def _w4_case(rng, kind, tall):
     for gi in range(k // g):
         want += (a[:, gi * g:(gi + 1) * g].astype(np.float64) @ q[gi * g:(gi + 1) * g].astype(np.float64)) * sc[gi]
     packed = dev(O.pack_int4(q))
+    bias = None
+    if kind == 'w4a16 with bias':
+        bias = (rng.integers(-40, 41, n) / 8.0).astype(np.float32)
     if kind == 'w4a16, decode layout':
         got = quant.symmetric_quant_matmul_w4a16_decode(dev(a, dt), quant.to_decode_layout_int4(packed), dev(sc, dt), g)
     else:
-        got = quant.symmetric_quant_matmul_w4a16(dev(a, dt), packed, dev(sc, dt), g)
+        got = quant.symmetric_quant_matmul_w4a16(dev(a, dt), packed, dev(sc, dt), g, bias=None if bias is None else dev(bias, dt))
     exp = O.to_bf16(want.astype(np.float32)) if dt == torch.bfloat16 else _f16(want).astype(np.float32)
+    if bias is not None:  # the second rounding
+        exp = O.to_bf16(exp + bias) if dt == torch.bfloat16 else _f16(exp + bias).astype(np.float32)
     return (m, k, n, g, str(dt)), np.array_equal(got.float().cpu().numpy(), exp.astype(np.float32))
 
 
@@ -127,7 +132,7 @@ def _f8_case(rng, kind, tall):
 
 
 FAMILIES = [('w8a16', _w8_case, 11), ('w8a16, K-contiguous weights', _w8_case, 12), ('w8a16 with bias', _w8_case, 13),
-            ('w4a16', _w4_case, 14), ('w4a16, decode layout', _w4_case, 15), ('matmul_f8', _f8_case, 16),
+            ('w4a16', _w4_case, 14), ('w4a16, decode layout', _w4_case, 15), ('w4a16 with bias', _w4_case, 18), ('matmul_f8', _f8_case, 16),
             ('matmul_f8_scaled', _f8_case, 17)]
 
 

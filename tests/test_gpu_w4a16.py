@@ -134,6 +134,51 @@ def test_decode_layout_exact_and_errors():
                                                   torch.zeros(2, 16, device='cuda', dtype=torch.bfloat16), 128)
 
 
+@pytest.mark.parametrize('m,k,n,g', [(1, 4096, 11008, 128), (16, 4096, 11008, 128), (3, 512, 272, 64), (20, 1024, 528, 128),
+                                     (1, 256, 40, 128),                     # N not a multiple of 16: the one-thread-per-element kernel
+                                     (48, 4096, 1024, 128), (300, 512, 544, 64), (512, 4096, 1024, 128), (768, 2048, 11008, 128)])
+@pytest.mark.parametrize('dtype', ['bfloat16', 'float16'])
+def test_bias_exact_and_the_bits_of_matmul_then_add(m, k, n, g, dtype):
+    """bias[n] of the output's type, added to the rounded result (two roundings). Small integers, power-of-two scales and
+    biases that are multiples of 1/8: integer arithmetic says what both roundings must give; and on random operands the
+    fused call returns the bits of the plain call followed by torch's add in the same type. Up to 32 rows the add rides
+    in the kernel's epilogue, above it follows the GEMM as a pass of its own."""
+    announce('w4a16 bias', m, k, n, g, dtype)
+    tdt = torch.bfloat16 if dtype == 'bfloat16' else torch.float16
+    rng = np.random.default_rng(m + n)
+    a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    q = rng.integers(-8, 8, (k, n)).astype(np.int8)
+    scales = (2.0 ** rng.integers(-3, 1, (k // g, n))).astype(np.float32)
+    bias = (rng.integers(-40, 41, n) / 8.0).astype(np.float32)
+    want = np.zeros((m, n))
+    for gi in range(k // g):
+        want += (a[:, gi * g:(gi + 1) * g].astype(np.float64) @ q[gi * g:(gi + 1) * g].astype(np.float64)) * scales[gi]
+    if dtype == 'bfloat16':
+        want = O.to_bf16(O.to_bf16(want.astype(np.float32)) + bias)
+    else:
+        with np.errstate(over='ignore'):
+            want = (want.astype(np.float32).astype(np.float16).astype(np.float32) + bias).astype(np.float16).astype(np.float32)
+    tp, ts, tb = dev(O.pack_int4(q)), dev(scales, tdt), dev(bias, tdt)
+    got = quant.symmetric_quant_matmul_w4a16(dev(a, tdt), tp, ts, g, bias=tb)
+    assert np.array_equal(got.float().cpu().numpy(), want)
+    # random operands: fused == plain + add, bit for bit
+    _, _, _, ta, tp, ts = _case(7, m, k, n, g, dtype)
+    tb = dev(np.random.default_rng(3).normal(0, 1, n).astype(np.float32), tdt)
+    fused = quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g, bias=tb)
+    plain = quant.symmetric_quant_matmul_w4a16(ta, tp, ts, g)
+    assert torch.equal(fused, plain + tb)
+
+
+def test_bias_argument_errors():
+    a = torch.zeros(2, 128, device='cuda', dtype=torch.bfloat16)
+    packed = torch.zeros(128, 8, device='cuda', dtype=torch.uint8)
+    scales = torch.zeros(1, 16, device='cuda', dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        quant.symmetric_quant_matmul_w4a16(a, packed, scales, 128, bias=torch.zeros(16, device='cuda', dtype=torch.float16))
+    with pytest.raises(ValueError):
+        quant.symmetric_quant_matmul_w4a16(a, packed, scales, 128, bias=torch.zeros(8, device='cuda', dtype=torch.bfloat16))
+
+
 def test_k_split_is_deterministic():
     m, k, n, g = 129, 4096, 512, 128
     announce('w4a16 k split twice', m, k, n)
