@@ -24,6 +24,11 @@ inline size_t skinny_lds_bytes(int m, int waves) { return size_t(waves) * m * kS
 struct bf16_biased_t {
     uint16_t bits;
 };
+// Output type of a float16 kernel whose caller gave no bias: the column factor only, one rounding (_Float16 itself stands for
+// the epilogue with both).
+struct f16_unbiased_t {
+    _Float16 v;
+};
 
 template <typename OutT>
 __device__ __forceinline__ OutT skinny_to_out(float v);
@@ -323,6 +328,7 @@ struct SkinnyTail {
     // bias keep the shorter epilogue: every instruction behind the last weight delays the kernel's end.)
     __device__ __forceinline__ OutT finish(float sum, int e) const {
         if constexpr (std::is_same<OutT, _Float16>::value) return scaled_biased_f16(sum, scale[e], bias[e]);
+        else if constexpr (std::is_same<OutT, f16_unbiased_t>::value) return f16_unbiased_t{_Float16(sum * scale[e])};
         else if constexpr (std::is_same<OutT, bf16_biased_t>::value) return bf16_biased_t{biased_bf16_bits(sum, bias[e])};
         else return skinny_to_out<OutT>(sum);
     }
@@ -359,15 +365,19 @@ struct SkinnyTail {
         const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(factors.bias), 0,
                                                                             factors.bias != nullptr ? n * 2 : 0, 0x00020000);
         const int off = int(out_col) * 2;
+        constexpr bool kBias = !std::is_same<OutT, f16_unbiased_t>::value;
         if constexpr (CW == 1) {
             scale_bits[0] = __builtin_amdgcn_raw_buffer_load_b16(rs, off, 0, 0);
-            bias_bits[0] = __builtin_amdgcn_raw_buffer_load_b16(rb, off, 0, 0);
+            if constexpr (kBias) bias_bits[0] = __builtin_amdgcn_raw_buffer_load_b16(rb, off, 0, 0);
         } else {  // 8-byte loads: vectors 8-byte aligned, n a multiple of 4
-            const auto q = __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, 0), b = __builtin_amdgcn_raw_buffer_load_b64(rb, off, 0, 0);
+            const auto q = __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, 0);
             scale_bits[0] = q[0];
             scale_bits[1] = q[1];
-            bias_bits[0] = b[0];
-            bias_bits[1] = b[1];
+            if constexpr (kBias) {
+                const auto b = __builtin_amdgcn_raw_buffer_load_b64(rb, off, 0, 0);
+                bias_bits[0] = b[0];
+                bias_bits[1] = b[1];
+            }
         }
     }
     __device__ __forceinline__ void use_factors() {
@@ -375,7 +385,7 @@ struct SkinnyTail {
         for (int e = 0; e < CW; ++e) {
             // the vectors have the output's type: float16, or bfloat16 bits
             const uint16_t sb = uint16_t(scale_bits[e >> 1] >> (16 * (e & 1))), bb = uint16_t(bias_bits[e >> 1] >> (16 * (e & 1)));
-            constexpr bool kHalf16 = std::is_same<OutT, _Float16>::value;
+            constexpr bool kHalf16 = std::is_same<OutT, _Float16>::value || std::is_same<OutT, f16_unbiased_t>::value;
             scale[e] = factors.scale != nullptr ? (kHalf16 ? f16_bits_to_f32(sb) : bf16_bits_to_f32(sb)) : 1.0f;
             bias[e] = factors.bias != nullptr ? (kHalf16 ? f16_bits_to_f32(bb) : bf16_bits_to_f32(bb)) : -0.0f;
         }

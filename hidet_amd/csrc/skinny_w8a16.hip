@@ -33,7 +33,7 @@ struct SkinnyStep {
     half8_t xa;
 };
 
-template <bool ALIGNED_A, int WAVES, int RING>
+template <bool ALIGNED_A, int WAVES, int RING, bool BIAS>
 __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_kernel(int ksteps, uint32_t ksteps_magic, int per_group, int longer, int splits, uint32_t splits_magic,
                                                                   const int8_t *__restrict__ w, const _Float16 *__restrict__ a,
                                                                   int64_t lda, int m, int k, int n, SkinnyPlanRest plan_rest,
@@ -151,8 +151,10 @@ __global__ __launch_bounds__(64 * WAVES) void skinny_w8a16_kernel(int ksteps, ui
 #pragma unroll
         for (int v = 0; v < 4; ++v) acc[t][v] -= 1152.0f * xsum[v];
     skinny_stash(acc, m, wave, red);
-    const SkinnyScale col_scale = {scale, bias};
-    skinny_tails<_Float16, WAVES>(plan, wk, roles, m, n, col_scale, c, mailbox, lost_flag, red);
+    // calls without a bias run the epilogue that never knew of one: every instruction behind the last weight counts
+    const SkinnyScale col_scale = {scale, BIAS ? bias : nullptr};
+    if constexpr (BIAS) skinny_tails<_Float16, WAVES>(plan, wk, roles, m, n, col_scale, c, mailbox, lost_flag, red);
+    else skinny_tails<f16_unbiased_t, WAVES>(plan, wk, roles, m, n, col_scale, reinterpret_cast<f16_unbiased_t *>(c), mailbox, lost_flag, red);
 }
 
 // Any shape the fast kernel cannot take (N not a multiple of 16, misaligned weights): one thread per
@@ -201,8 +203,13 @@ void skinny_w8a16_launch(const void *a, const void *w, const void *scale, const 
                    static_cast<const int8_t *>(w), ap, lda, mt, int(k), int(n), static_cast<SkinnyPlanRest>(plan),
                    static_cast<const _Float16 *>(scale), static_cast<const _Float16 *>(bias), cp, ws.mailbox, lost_flag);
         };
-        if (aligned_a) go(skinny_w8a16_kernel<true, waves, kRing>);
-        else go(skinny_w8a16_kernel<false, waves, kRing>);
+        if (bias != nullptr) {
+            if (aligned_a) go(skinny_w8a16_kernel<true, waves, kRing, true>);
+            else go(skinny_w8a16_kernel<false, waves, kRing, true>);
+        } else {
+            if (aligned_a) go(skinny_w8a16_kernel<true, waves, kRing, false>);
+            else go(skinny_w8a16_kernel<false, waves, kRing, false>);
+        }
     }
 }
 
